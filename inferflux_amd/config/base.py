@@ -83,6 +83,11 @@ class ModelConfig:
     def validate(self) -> None:
         raise NotImplementedError
 
+    def with_tensor_shapes(self, shapes: Mapping[str, Tuple[int, ...]]) -> "ModelConfig":
+        """The config completed by the sizes that its file leaves to the tensors' shapes (name -> shape of every tensor
+        of the model folder).  Most files name every size: they return themselves."""
+        return self
+
     def save(self, folder: str) -> None:
         os.makedirs(folder, exist_ok=True)
         with open(os.path.join(folder, "config.json"), "w") as f:

@@ -69,7 +69,19 @@ def config_from_dict(d: Mapping[str, Any]) -> ModelConfig:
 
 
 def load_config(folder: str) -> ModelConfig:
-    return config_from_dict(read_config_json(folder))
+    """The typed config of a model folder.  A config whose file leaves a size to a tensor's shape is completed from the
+    headers of the folder's weight files (no tensor is read)."""
+    cfg = config_from_dict(read_config_json(folder))
+    if type(cfg).with_tensor_shapes is not ModelConfig.with_tensor_shapes:
+        from ..weights.safetensors_io import open_model_files
+        files = open_model_files(folder)
+        try:
+            shapes = {n: tuple(f.shape(n)) for f in files for n in f.names()}
+        finally:
+            for f in files:
+                f.close()
+        cfg = cfg.with_tensor_shapes(shapes)
+    return cfg
 
 
 def plan_for(config: ModelConfig):

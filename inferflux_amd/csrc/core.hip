@@ -386,13 +386,18 @@ struct RopeArgs {
   const void* v_first;   // [T, nKV * dv] of the activation type: v <- (1 - v_mix) v + v_mix v_first before the cache write
   float v_mix;
   void* v_out;           // [T, nKV * dv]: the values as projected (with bias, before any mixing), for later layers to mix in
+  const void* q_norm_w;  // [d]: before the rotation every q head becomes x / sqrt(mean(x^2) + pre_norm_eps) * q_norm_w
+  const void* k_norm_w;  // [d]: the same for every k head (both or neither)
+  int pre_norm_dtype;
+  float pre_norm_eps;
+  int extra_cols;        // further columns at the end of a row that this kernel does not read (another kernel's)
 };
 
 template <typename T>
 __global__ __launch_bounds__(64) void rope_append_kernel(RopeArgs a) {
   const int t = blockIdx.x, head = blockIdx.y;
   const int d = a.d, dv = a.dv, half = d / 2, rot_half = a.rope_style != 0 ? a.rotary_dim / 2 : 0;
-  const int q_width = a.nH * d, kv_width = a.nKV * d, row_width = q_width + kv_width + a.nKV * dv + a.gate_cols;
+  const int q_width = a.nH * d, kv_width = a.nKV * d, row_width = q_width + kv_width + a.nKV * dv + a.gate_cols + a.extra_cols;
   const T* row = (const T*)a.qkv + (size_t)t * row_width;
   const float* part = (const float*)a.qkv + (size_t)t * row_width;
   // Elements i0 and i1 of the row; partial sums are added in slice order, eight slices of both elements asked for
@@ -427,6 +432,21 @@ __global__ __launch_bounds__(64) void rope_append_kernel(RopeArgs a) {
     if (!is_q && slot < 0) return;
     T* dst = is_q ? (T*)a.q_out + (size_t)t * q_width + col
                   : (T*)a.k_cache + (((size_t)page * a.nKV + (head - a.nH)) * a.page_size + off) * d;
+    const void* pre_w = is_q ? a.q_norm_w : a.k_norm_w;
+    float pre_inv = 1.f;
+    if (pre_w) {             // the head's root mean square before the rotation (the block is one wave)
+      float ss = 0.f;
+      for (int p = threadIdx.x; p < half; p += blockDim.x) {
+        float x0, x1;
+        in2(col + 2 * p, col + 2 * p + 1, x0, x1);
+        if (a.bias) {
+          x0 += load_dyn(a.bias, a.bias_dtype, col + 2 * p);
+          x1 += load_dyn(a.bias, a.bias_dtype, col + 2 * p + 1);
+        }
+        ss += x0 * x0 + x1 * x1;
+      }
+      pre_inv = rsqrtf(wave_sum(ss) / (float)d + a.pre_norm_eps);
+    }
     // pair p of the head with bias and rotation: elements i0, i1 and their values
     auto pair = [&](int p, int& i0, int& i1, float& y0, float& y1) {
       const bool rotate = p < rot_half;
@@ -441,6 +461,10 @@ __global__ __launch_bounds__(64) void rope_append_kernel(RopeArgs a) {
       if (a.bias) {
         x0 += load_dyn(a.bias, a.bias_dtype, col + i0);
         x1 += load_dyn(a.bias, a.bias_dtype, col + i1);
+      }
+      if (pre_w) {
+        x0 *= pre_inv * load_dyn(pre_w, a.pre_norm_dtype, i0);
+        x1 *= pre_inv * load_dyn(pre_w, a.pre_norm_dtype, i1);
       }
       y0 = x0; y1 = x1;
       if (rotate) {
@@ -587,7 +611,7 @@ __global__ __launch_bounds__(256) void rope_append_vec_kernel(RopeArgs a, int T,
 // above, dv wide, mixed and handed on where asked.
 __global__ __launch_bounds__(256) void rope_append_vec_x_kernel(RopeArgs a, int T, int n_qk_blocks) {
   const int d = a.d, dv = a.dv, rot = a.rope_style != 0 ? a.rotary_dim : 0;
-  const int q_width = a.nH * d, kv_width = a.nKV * d, v_width = a.nKV * dv, row_width = q_width + kv_width + v_width + a.gate_cols;
+  const int q_width = a.nH * d, kv_width = a.nKV * d, v_width = a.nKV * dv, row_width = q_width + kv_width + v_width + a.gate_cols + a.extra_cols;
   const bf16_t* qkv = (const bf16_t*)a.qkv;
   const bf16_t* bias = (const bf16_t*)a.bias;
   if ((int)blockIdx.x < n_qk_blocks) {
@@ -606,6 +630,17 @@ __global__ __launch_bounds__(256) void rope_append_vec_x_kernel(RopeArgs a, int 
       const rope_bf16x8 b0 = *(const rope_bf16x8*)(bias + head * d + first), b1 = *(const rope_bf16x8*)(bias + head * d + second);
 #pragma unroll
       for (int e = 0; e < 8; ++e) { f0[e] += (float)b0[e]; f1[e] += (float)b1[e]; }
+    }
+    const bf16_t* pre_w = (const bf16_t*)(head < a.nH ? a.q_norm_w : a.k_norm_w);
+    if (pre_w) {             // the head's root mean square before the rotation, then the norm's weight
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += f0[e] * f0[e] + f1[e] * f1[e];
+      for (int o = per_head / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, WAVE);
+      const float pre_inv = rsqrtf(ss / (float)d + a.pre_norm_eps);
+      const rope_bf16x8 w0 = *(const rope_bf16x8*)(pre_w + first), w1 = *(const rope_bf16x8*)(pre_w + second);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { f0[e] *= pre_inv * (float)w0[e]; f1[e] *= pre_inv * (float)w1[e]; }
     }
     if (rotate) {
       const float* cs = a.cs + (size_t)t * (rot / 2) + 8 * j;
@@ -696,7 +731,9 @@ extern "C" int ifx_rope_append(const void* qkv, int dtype, const void* bias, int
                                const float* cs, const float* sn, int rope_style, int rotary_dim, int T, int nH,
                                int nKV, int d, int page_size, void* q_out, void* k_cache, void* v_cache, int n_slices,
                                long long slice_stride, int dv, int gate_cols, float* gate_out, int unit_norm, float norm_eps,
-                               const void* v_first, float v_mix, void* v_out, void* stream) {
+                               const void* v_first, float v_mix, void* v_out, const void* q_norm_w, const void* k_norm_w,
+                               int pre_norm_dtype, float pre_norm_eps, int extra_cols, void* stream) {
+  IFX_REQUIRE((q_norm_w != nullptr) == (k_norm_w != nullptr) && extra_cols >= 0, "rope_append: norms for q and k come together");
   IFX_REQUIRE(n_slices >= 1 && (n_slices == 1 || slice_stride > 0), "rope_append: %d slices, %lld apart", n_slices, slice_stride);
   IFX_REQUIRE(T >= 0 && nH > 0 && nKV >= 0 && d > 0 && d % 2 == 0 && dv > 0, "rope_append: bad sizes T=%d nH=%d nKV=%d d=%d dv=%d", T, nH, nKV, d, dv);
   IFX_REQUIRE(rope_style >= 0 && rope_style <= 2, "rope_append: unknown rope style %d", rope_style);
@@ -708,8 +745,9 @@ extern "C" int ifx_rope_append(const void* qkv, int dtype, const void* bias, int
   IFX_REQUIRE(gate_cols == 0 || (gate_cols == nH && gate_out), "rope_append: %d gate columns for %d heads", gate_cols, nH);
   IFX_REQUIRE(!(v_first || v_out) || nKV > 0, "rope_append: values to mix or to hand on, but no kv heads");
   RopeArgs a{qkv, n_slices, (size_t)slice_stride, bias, bias_dtype, slots, cs, sn, rope_style, rotary_dim, nH, nKV, d, page_size,
-             q_out, k_cache, v_cache, dv, gate_cols, gate_out, unit_norm, norm_eps, v_first, v_mix, v_out};
-  const bool extras = gate_cols || unit_norm || v_first || v_out;
+             q_out, k_cache, v_cache, dv, gate_cols, gate_out, unit_norm, norm_eps, v_first, v_mix, v_out,
+             q_norm_w, k_norm_w, pre_norm_dtype, pre_norm_eps, extra_cols};
+  const bool extras = gate_cols || unit_norm || v_first || v_out || q_norm_w || extra_cols;
   hipStream_t s = (hipStream_t)stream;
   // (a few tokens are quicker with one small block per token and head: nothing waits on a loop over tokens)
   if (!extras && dv == d && T >= 128 && n_slices == 1 && dtype == DT_BF16 && rope_style == 1 && rotary_dim == d && d % 16 == 0 && (!bias || bias_dtype == DT_BF16) &&
@@ -722,7 +760,8 @@ extern "C" int ifx_rope_append(const void* qkv, int dtype, const void* bias, int
   }
   const int rot = rope_style != 0 ? rotary_dim : 0;
   if (extras && T >= 128 && n_slices == 1 && dtype == DT_BF16 && rope_style <= 1 && (d == 16 || d == 32 || d == 64 || d == 128) &&
-      rot % 16 == 0 && (nH * d + nKV * (d + dv) + gate_cols) % 8 == 0 && (!bias || bias_dtype == DT_BF16) &&
+      rot % 16 == 0 && (nH * d + nKV * (d + dv) + gate_cols + extra_cols) % 8 == 0 && (!bias || bias_dtype == DT_BF16) &&
+      (!q_norm_w || pre_norm_dtype == DT_BF16) &&
       (!slots || page_size % 8 == 0) && (slots || (!v_first && !v_out))) {
     const size_t qk_threads = (size_t)T * (nH + (slots ? nKV : 0)) * (d / 16);
     const size_t v_threads = (slots || v_out) ? (size_t)((T + 7) / 8) * nKV * dv : 0;

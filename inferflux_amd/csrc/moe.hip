@@ -67,6 +67,7 @@ struct RouteArgs {
   const void* h; const void* w; const float* z; int* ids; float* weights;
   int T, K, E, top, groups, keep, group_top, softmax, renorm;
   float scale;
+  const float* bias;     // [E] added to the logits, or null
 };
 
 template <typename T>
@@ -103,6 +104,10 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(RouteArgs a) {
     }
   }
   __syncthreads();
+  if (a.bias) {
+    for (int e = threadIdx.x; e < a.E; e += blockDim.x) s[e] += a.bias[e];
+    __syncthreads();
+  }
   if (a.softmax) {
     float m = -INFINITY;
     for (int e = threadIdx.x; e < a.E; e += blockDim.x) m = fmaxf(m, s[e]);
@@ -162,14 +167,14 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(RouteArgs a) {
 }
 
 extern "C" int ifx_moe_route(const void* h, const void* w, int dtype, const float* z, int* ids, float* weights, int T, int K, int E,
-                             int top, int groups, int keep, int group_top, int softmax, int renorm, float scale, void* stream) {
+                             int top, int groups, int keep, int group_top, int softmax, int renorm, float scale, const float* bias, void* stream) {
   IFX_REQUIRE(z || (h && w), "moe_route: neither logits nor the rows and the router's weight");
   IFX_REQUIRE(T >= 0 && K > 0 && E > 0 && E <= MAX_EXPERTS, "moe_route: %d experts (at most %d), K=%d", E, MAX_EXPERTS, K);
   IFX_REQUIRE(groups > 0 && E % groups == 0 && keep > 0 && keep <= groups, "moe_route: %d experts in %d groups of which %d are kept", E, groups, keep);
   IFX_REQUIRE(group_top > 0 && group_top <= 8, "moe_route: a group's score sums its %d largest (1-8)", group_top);
   IFX_REQUIRE(top > 0 && top <= MAX_TOP && top <= keep * (E / groups), "moe_route: top %d of %d x %d experts", top, keep, E / groups);
   if (T == 0) return 0;
-  RouteArgs a{h, w, z, ids, weights, T, K, E, top, groups, keep, group_top, softmax, renorm, scale};
+  RouteArgs a{h, w, z, ids, weights, T, K, E, top, groups, keep, group_top, softmax, renorm, scale, bias};
   // a wave takes four experts at a time: as many waves as that takes, up to 16 (the scores are a chain of trips to memory otherwise)
   const int threads = z ? WAVE * (E <= 64 ? 1 : 4) : WAVE * (E <= 16 ? 4 : (E <= 32 ? 8 : 16));
   hipStream_t s = (hipStream_t)stream;

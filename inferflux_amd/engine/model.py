@@ -123,6 +123,10 @@ class Model:
                 residual, pending = block.forward(residual, pending, ctx, storage.binding(i), following=following)
             else:
                 residual, pending = block.forward(residual, pending, ctx, storage.binding(i))
+        if schedule:
+            close = getattr(self.blocks[schedule[-1].layer], "close_stream", None)
+            if close is not None:                    # (an arrangement with several streams hands back the one the final norm reads)
+                residual, pending = close(residual, pending, ctx)
         if getattr(pending, "in_stream", False):     # (a block's hand-over to its like; the stream holds everything)
             pending = None
         if ctx.n_logit_rows == 0:

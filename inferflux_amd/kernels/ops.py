@@ -58,6 +58,9 @@ def module_variants() -> Iterable[Tuple[str, Variant]]:
     yield ("latent", ())
     yield ("moe", ())
     yield ("ssm", ())
+    yield ("gla", ())
+    yield ("hyper", ())
+    yield ("rowwise", ())
     yield ("grouped_gemm", ())
     yield ("ceilings", ())            # measurement only: what the memory gives a kernel that just reads
     for d in MFMA_HEAD_DIMS_PREBUILT:
@@ -204,8 +207,13 @@ def rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], slots: Optional
                 rotary_dim: int, n_heads: int, n_kv_heads: int, head_dim: int,
                 k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], page_size: int,
                 v_head_dim: Optional[int] = None, unit_norm_eps: Optional[float] = None, gate_out: Optional[torch.Tensor] = None,
-                v_first: Optional[torch.Tensor] = None, v_mix: float = 0.0, v_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                v_first: Optional[torch.Tensor] = None, v_mix: float = 0.0, v_out: Optional[torch.Tensor] = None,
+                qk_norm: Optional[Tuple[torch.Tensor, torch.Tensor, float]] = None, extra_cols: int = 0) -> torch.Tensor:
     """Bias, rotation and cache write of one step's projections; returns q [T, n_heads, head_dim].
+
+    ``qk_norm`` (q weight [head_dim], k weight [head_dim], eps): before the rotation every q and k head becomes
+    x / sqrt(mean(x^2) + eps) * weight.  ``extra_cols``: further columns at the end of every row of ``qkv`` that belong
+    to another kernel (a gate that is applied elsewhere).
 
     Optionally: ``unit_norm_eps`` divides every q and k head by its root mean square (eps inside the root) after the
     rotation; ``gate_out`` (float32 [T, n_heads]) receives sigmoid(x + bias) of n_heads further columns behind q, k and v
@@ -220,7 +228,7 @@ def rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], slots: Optional
     T = qkv.shape[0]
     dv = head_dim if v_head_dim is None else int(v_head_dim)
     gate_cols = n_heads if gate_out is not None else 0
-    width = (n_heads + n_kv_heads) * head_dim + n_kv_heads * dv + gate_cols
+    width = (n_heads + n_kv_heads) * head_dim + n_kv_heads * dv + gate_cols + int(extra_cols)
     n_slices = 1
     if isinstance(qkv, SliceSums):                  # partial sums: the kernel adds them in slice order
         _check(qkv.parts, "qkv", (None, T, width), torch.float32)
@@ -244,14 +252,20 @@ def rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], slots: Optional
     for t, nm in ((v_first, "v_first"), (v_out, "v_out")):
         if t is not None:
             _check(t, nm, (T, n_kv_heads * dv), dtype)
+    qn = kn = None
+    if qk_norm is not None:
+        qn, kn, pre_eps = qk_norm
+        _check(qn, "q norm weight", (head_dim,))
+        _check(kn, "k norm weight", (head_dim,), qn.dtype)
     q = torch.empty((T, n_heads, head_dim), dtype=dtype, device=qkv.device)
     _call(load_module("core"), "ifx_rope_append",
-          (P, I, P, I, P, P, P, I, I, I, I, I, I, I, P, P, P, I, LL, I, I, P, I, F, P, F, P, P),
+          (P, I, P, I, P, P, P, I, I, I, I, I, I, I, P, P, P, I, LL, I, I, P, I, F, P, F, P, P, P, I, F, I, P),
           qkv.data_ptr(), _DT[dtype], _ptr(bias), _dt(bias) if bias is not None else 0, _ptr(slots),
           _ptr(cos) if rope_style != ROPE_NONE else 0, _ptr(sin) if rope_style != ROPE_NONE else 0, rope_style,
           rotary_dim, T, n_heads, n_kv_heads, head_dim, page_size, q.data_ptr(), _ptr(k_cache), _ptr(v_cache),
           n_slices, T * width, dv, gate_cols, _ptr(gate_out), 1 if unit_norm_eps is not None else 0,
-          float(unit_norm_eps or 0.0), _ptr(v_first), float(v_mix), _ptr(v_out), _stream())
+          float(unit_norm_eps or 0.0), _ptr(v_first), float(v_mix), _ptr(v_out), _ptr(qn), _ptr(kn),
+          _dt(qn) if qn is not None else 0, float(pre_eps) if qn is not None else 0.0, int(extra_cols), _stream())
     return q
 
 
@@ -396,12 +410,12 @@ ROUTE_FUSED_MAX_ROWS = 16       # rows up to which the router's kernel forms the
 
 
 def moe_route(h: torch.Tensor, router, top: int, groups: int = 1, keep_groups: int = 1, group_top: int = 2,
-              softmax: bool = False, renormalize: bool = False, scale: float = 1.0):
+              softmax: bool = False, renormalize: bool = False, scale: float = 1.0, bias: Optional[torch.Tensor] = None):
     """The router of a mixture of experts, in float: scores of ``router`` [E, K] (a tensor or a ``LinearWeight``) times the
     rows of ``h`` [T, K] through a sigmoid (or a softmax over the experts), the ``top`` highest among the experts of the best
     ``keep_groups`` of ``groups`` equal groups of neighbours (a group scores the sum of its ``group_top`` highest).  Returns
     (ids int32 [T, top], weights float32 [T, top]): the chosen scores, divided by their sum with ``renormalize``, times
-    ``scale``.  Up to ``ROUTE_FUSED_MAX_ROWS`` rows the kernel forms the logits itself; more rows in bfloat16 get them from
+    ``scale``.  ``bias`` float32 [E] is added to the logits before anything else.  Up to ``ROUTE_FUSED_MAX_ROWS`` rows the kernel forms the logits itself; more rows in bfloat16 get them from
     ``linear`` with float32 sums and output."""
     _check(h, "h", (None, None))
     T, K = h.shape
@@ -412,9 +426,11 @@ def moe_route(h: torch.Tensor, router, top: int, groups: int = 1, keep_groups: i
     z = linear(h, router, out_dtype=torch.float32) if (T > ROUTE_FUSED_MAX_ROWS and h.dtype == torch.bfloat16) else None
     ids = torch.empty((T, top), dtype=torch.int32, device=h.device)
     weights = torch.empty((T, top), dtype=torch.float32, device=h.device)
-    _call(load_module("moe"), "ifx_moe_route", (P, P, I, P, P, P, I, I, I, I, I, I, I, I, I, F, P),
+    if bias is not None:
+        _check(bias, "bias", (E,), torch.float32)
+    _call(load_module("moe"), "ifx_moe_route", (P, P, I, P, P, P, I, I, I, I, I, I, I, I, I, F, P, P),
           h.data_ptr(), rows.data_ptr(), _dt(h), _ptr(z), ids.data_ptr(), weights.data_ptr(), T, K, E, top, groups, keep_groups,
-          group_top, 1 if softmax else 0, 1 if renormalize else 0, float(scale), _stream())
+          group_top, 1 if softmax else 0, 1 if renormalize else 0, float(scale), _ptr(bias), _stream())
     return ids, weights
 
 
@@ -1153,6 +1169,193 @@ def scan_chunks(q_start, q_len, chunk: int, device) -> Dict[str, object]:
     w = n + -n % 4
     return {"req": packed[:n], "t0": packed[w:w + n], "len": packed[2 * w:2 * w + n], "req_chunk0": packed[3 * w:3 * w + len(first)],
             "rows": int(chunk)}       # (the most rows a chunk has: the kernels keep a chunk's B and C in LDS)
+
+
+# ----------------------------------------------------------------------------------------
+GLA_THREAD_CHANNELS = ((16, 512), (32, 1024), (64, 512), (128, 256))   # channels of S a thread may hold, and the threads a workgroup may then have
+
+
+def gla_layout(d: int, dv: int) -> Tuple[int, int]:
+    """(channels a thread holds, threads per column) for a head of d key channels and dv values: the first pairing whose
+    workgroup (dv columns times the threads of a column) fits.  A request's S takes heads * dv * parts * channels floats."""
+    for dp, max_threads in GLA_THREAD_CHANNELS:
+        parts = 1
+        while parts * dp < d:
+            parts *= 2
+        if parts <= 64 and dv * parts <= max_threads:
+            return dp, parts
+    raise KernelError(f"gla: a head of {d} key channels and {dv} values does not fit a workgroup")
+
+
+def gla_state_floats(n_heads: int, d: int, dv: int) -> int:
+    dp, parts = gla_layout(d, dv)
+    return n_heads * dv * parts * dp
+
+
+def gla_scan(rows: torch.Tensor, cols: Tuple[int, int, int, int], z: torch.Tensor, z_bias: Optional[torch.Tensor], tau: float,
+             q_scale: float, norm_weight: torch.Tensor, eps: float, n_heads: int, d: int, dv: int, state: torch.Tensor,
+             state_offset: int, q_start: torch.Tensor, q_len: torch.Tensor, slots: torch.Tensor,
+             chunks: Optional[Dict[str, object]] = None) -> torch.Tensor:
+    """Gated linear attention over each request's rows, with the output's norm and gate:
+    alpha = sigmoid(z + z_bias) ^ (1 / tau) per key channel; per head S <- diag(alpha) S + k v^T; o = S^T q * q_scale;
+    y = o / sqrt(mean(o^2) + eps) * norm_weight * silu(g).  ``rows`` [T, ld] holds q, k (n_heads * d each), v and g
+    (n_heads * dv each) at the columns ``cols`` = (q, k, v, g); ``z`` float32 [T, n_heads * d]; ``state`` float32
+    [slots, n] with a request's S (``gla_state_floats`` numbers, laid out for the kernel) at ``state_offset`` of its row.
+    Decays, S, o, norm and gate are float.  Returns y [T, n_heads * dv] in the rows' type.
+
+    ``chunks`` (from ``scan_chunks``): the requests' rows cut into chunks that run side by side, first from a zero state,
+    then from the state the chunks before leave (the recurrence is linear in S); the same function up to the rounding of
+    float sums taken in another order."""
+    _check(rows, "rows", (None, None))
+    T, ld = rows.shape
+    HD, HV = n_heads * d, n_heads * dv
+    q_col, k_col, v_col, g_col = (int(c) for c in cols)
+    for c, w, nm in ((q_col, HD, "q"), (k_col, HD, "k"), (v_col, HV, "v"), (g_col, HV, "g")):
+        if c < 0 or c + w > ld:
+            raise KernelError(f"gla_scan: the {nm} columns {c}..{c + w} lie outside rows of {ld}")
+    _check(z, "z", (T, HD), torch.float32)
+    if z_bias is not None:
+        _check(z_bias, "z_bias", (HD,), torch.float32)
+    _check(norm_weight, "norm_weight", (dv,))
+    _check(state, "state", (None, None), torch.float32)
+    R = q_start.shape[0]
+    for t, nm in ((q_start, "q_start"), (q_len, "q_len"), (slots, "slots")):
+        _check(t, nm, (R,), torch.int32)
+    dp, parts = gla_layout(d, dv)
+    out = torch.empty((T, HV), dtype=rows.dtype, device=rows.device)
+    n_chunks, lists = 0, (0, 0, 0, 0, 0, 0)
+    if chunks is not None:
+        n_chunks = chunks["req"].shape[0]
+        for nm in ("req", "t0", "len"):
+            _check(chunks[nm], f"chunks.{nm}", (n_chunks,), torch.int32)
+        _check(chunks["req_chunk0"], "chunks.req_chunk0", (R + 1,), torch.int32)
+        chunk_state = torch.empty((n_chunks, HV * parts * dp), dtype=torch.float32, device=rows.device)
+        chunk_loga = torch.empty((n_chunks, HD), dtype=torch.float32, device=rows.device)
+        lists = (chunks["req"].data_ptr(), chunks["t0"].data_ptr(), chunks["len"].data_ptr(), chunks["req_chunk0"].data_ptr(),
+                 chunk_state.data_ptr(), chunk_loga.data_ptr())
+    _call(load_module("gla"), "ifx_gla_scan",
+          (P, I, I, I, I, I, I, P, P, F, F, F, P, I, P, LL, LL, P, P, P, P, I, I, I, I, I, I, I, I, P, P, P, P, P, P, P),
+          rows.data_ptr(), _dt(rows), ld, q_col, k_col, v_col, g_col, z.data_ptr(), _ptr(z_bias), 1.0 / float(tau), float(q_scale),
+          float(eps), norm_weight.data_ptr(), _dt(norm_weight), state.data_ptr(), state.shape[1], int(state_offset),
+          q_start.data_ptr(), q_len.data_ptr(), slots.data_ptr(), out.data_ptr(), T, R, n_heads, d, dv, dp, parts, n_chunks,
+          *lists, _stream())
+    return out
+
+
+HYPER_MAX_STREAMS = 8
+
+
+def hyper_step(src: torch.Tensor, n_streams: int, y=None, mix: Optional[torch.Tensor] = None, out_weights: Optional[torch.Tensor] = None,
+               in_weights: Optional[torch.Tensor] = None, norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0,
+               out_dtype: Optional[torch.dtype] = None, y_scale: float = 1.0):
+    """One step of hyper-connections on the streams of a step's rows, in float.
+
+    ``src`` float32: the streams [T, S, H], or one stream [T, H] that all S start as.  With ``y`` [T, H] (a tensor of any
+    activation type or ``SliceSums``) the streams become x_t <- sum_s mix[s, t] x_s + out_weights[t] * y * y_scale, in
+    place (copies of a single stream are written to a new tensor).  With ``in_weights`` the sub-block that follows reads
+    u = sum_t in_weights[t] x_t of the new streams: returned normalised, u / sqrt(mean(u^2) + eps) * norm_weight in
+    ``out_dtype``, or as it is in float32 without ``norm_weight``.  Returns (streams, rows or None)."""
+    S = int(n_streams)
+    single = src.dim() == 2
+    if single:
+        _check(src, "src", (None, None), torch.float32)
+        T, H = src.shape
+    else:
+        _check(src, "src", (None, S, None), torch.float32)
+        T, _, H = src.shape
+    if not 0 < S <= HYPER_MAX_STREAMS:
+        raise KernelError(f"hyper_step: {S} streams (1 to {HYPER_MAX_STREAMS})")
+    for t, nm, shape in ((mix, "mix", (S, S)), (out_weights, "out_weights", (S,)), (in_weights, "in_weights", (S,))):
+        if t is not None:
+            _check(t, nm, shape, torch.float32)
+    n_slices, stride, y_ptr, y_dt = 1, 0, 0, 0
+    if y is not None:
+        if mix is None or out_weights is None:
+            raise KernelError("hyper_step: an update needs the mixing matrix and the output weights")
+        if isinstance(y, SliceSums):
+            _check(y.parts, "y", (None, T, H), torch.float32)
+            n_slices, stride, y_ptr, y_dt = y.parts.shape[0], T * H, y.parts.data_ptr(), DT_F32
+        else:
+            _check(y, "y", (T, H))
+            y_ptr, y_dt = y.data_ptr(), _dt(y)
+    dst = torch.empty((T, S, H), dtype=torch.float32, device=src.device) if single else src
+    rows = None
+    if in_weights is not None:
+        if norm_weight is not None:
+            _check(norm_weight, "norm_weight", (H,))
+            rows = torch.empty((T, H), dtype=out_dtype or torch.float32, device=src.device)
+        else:
+            rows = torch.empty((T, H), dtype=torch.float32, device=src.device)
+    _call(load_module("hyper"), "ifx_hyper_step", (P, I, P, P, I, I, LL, F, P, P, P, P, I, F, P, I, I, I, I, P),
+          src.data_ptr(), 1 if single else 0, dst.data_ptr(), y_ptr, y_dt, n_slices, stride, float(y_scale), _ptr(mix), _ptr(out_weights),
+          _ptr(in_weights), _ptr(norm_weight), _dt(norm_weight) if norm_weight is not None else 0, float(eps), _ptr(rows),
+          _DT[rows.dtype] if rows is not None else 0, T, S, H, _stream())
+    return dst, rows
+
+
+def linear_act(x, weight, act: int) -> torch.Tensor:
+    """act(x W^T) for a feed-forward without a gate (``act``: ACT_SILU or ACT_GELU_TANH, formed in float on the product's
+    output)."""
+    return activation(linear(x, weight), act)
+
+
+def activation(x: torch.Tensor, act: int) -> torch.Tensor:
+    """act(x) element by element in float: ACT_SILU or ACT_GELU_TANH (a feed-forward without a gate)."""
+    _check(x, "x")
+    out = torch.empty_like(x)
+    _call(load_module("rowwise"), "ifx_activation", (P, P, I, LL, I, P), x.data_ptr(), out.data_ptr(), _dt(x), x.numel(), int(act), _stream())
+    return out
+
+
+def sigmoid_gate(x: torch.Tensor, rows, g_col: int) -> torch.Tensor:
+    """x [T, C] times sigmoid of the columns ``g_col`` .. ``g_col`` + C - 1 of ``rows`` [T, ld] (x's type, or ``SliceSums``),
+    element by element, the sigmoid in float."""
+    _check(x, "x", (None, None))
+    T, C = x.shape
+    n_slices, stride = 1, 0
+    if isinstance(rows, SliceSums):
+        _check(rows.parts, "rows", (None, T, None), torch.float32)
+        n_slices, ld, stride, ptr = rows.parts.shape[0], rows.parts.shape[2], T * rows.parts.shape[2], rows.parts.data_ptr()
+    else:
+        _check(rows, "rows", (T, None), x.dtype)
+        ld, ptr = rows.shape[1], rows.data_ptr()
+    if g_col < 0 or g_col + C > ld:
+        raise KernelError(f"sigmoid_gate: columns {g_col}..{g_col + C} lie outside rows of {ld}")
+    out = torch.empty_like(x)
+    _call(load_module("rowwise"), "ifx_sigmoid_gate", (P, P, I, I, I, LL, P, I, I, I, P),
+          x.data_ptr(), ptr, ld, int(g_col), n_slices, stride, out.data_ptr(), _dt(x), T, C, _stream())
+    return out
+
+
+def gated_add(base, extra, h: torch.Tensor, gate_weight: torch.Tensor) -> torch.Tensor:
+    """base + sigmoid(h . gate_weight) * extra row by row: ``base`` and ``extra`` [T, N] (h's type, or ``SliceSums``, which are
+    added in slice order), ``h`` [T, K], ``gate_weight`` [K] (one number per row, formed in float).  Returns [T, N] in h's type."""
+    _check(h, "h", (None, None))
+    T, K = h.shape
+    _check(gate_weight, "gate_weight", (K,), h.dtype)
+
+    def operand(v, nm):
+        if isinstance(v, SliceSums):
+            _check(v.parts, nm, (None, T, None), torch.float32)
+            return v.parts.data_ptr(), 1, v.parts.shape[0], T * v.parts.shape[2], v.parts.shape[2]
+        _check(v, nm, (T, None), h.dtype)
+        return v.data_ptr(), 1 if v.dtype == torch.float32 else 0, 1, 0, v.shape[1]
+
+    bp, bf, bn, bs, N = operand(base, "base")
+    ep, ef, en, es, N2 = operand(extra, "extra")
+    if N != N2:
+        raise KernelError(f"gated_add: base is {N} wide, extra {N2}")
+    out = torch.empty((T, N), dtype=h.dtype, device=h.device)
+    _call(load_module("rowwise"), "ifx_gated_add", (P, I, I, LL, P, I, I, LL, P, P, I, P, I, I, I, P),
+          bp, bf, bn, bs, ep, ef, en, es, h.data_ptr(), gate_weight.data_ptr(), K, out.data_ptr(), _dt(h), T, N, _stream())
+    return out
+
+
+def scale_softcap(logits: torch.Tensor, scale: float = 1.0, cap: float = 0.0) -> torch.Tensor:
+    """In place on float32 ``logits``: x <- x * scale, then (cap > 0) x <- cap * tanh(x / cap)."""
+    _check(logits, "logits", None, torch.float32)
+    _call(load_module("rowwise"), "ifx_scale_softcap", (P, LL, F, F, P), logits.data_ptr(), logits.numel(), float(scale), float(cap or 0.0), _stream())
+    return logits
 
 
 WIDE_MAX_K_DIM, WIDE_MAX_V_DIM = 1024, 512

@@ -19,13 +19,16 @@ Optional mechanisms, each a constructor argument that is off by default:
                       (exp(sink) + sum_j exp(s_j)); with 0 that is "one added to the denominator".
   ``unit_norm_eps``   after the rotation every q and k head is divided by its root mean square (eps inside the root; an
                       RMS norm without weight).
-  ``output_gate``     head h's output is multiplied by sigmoid(W_g x)_h before the output projection (W_g [heads, H], a
-                      further block of rows of the fused projection).
+  ``output_gate``     True: head h's output is multiplied by sigmoid(W_g x)_h before the output projection (W_g [heads, H], a
+                      further block of rows of the fused projection).  "elementwise": the concatenated heads are multiplied
+                      element by element with sigmoid(W_g x) (W_g [heads * v_head_dim, H]).
+  ``qk_norm_eps``     before the rotation every q and k head becomes x / sqrt(mean(x^2) + eps) * w, with one weight of
+                      head_dim for all q heads ("q_norm") and one for all k heads ("k_norm").
   ``value_mix``       "source": this layer hands the step's values (as projected) on to the layers after it; "mix": this
                       layer caches v <- (1 - lambda) v + lambda v_source instead of its own, lambda a scalar tensor.  The
                       layers must agree in kv heads and value width.
   ``tensors``         full names of the tensors in the model file ("q", "k", "v", "o", "q_bias", "k_bias", "v_bias", "gate",
-                      "mix") where they are not ``<name>.q_proj.weight`` and so on.
+                      "mix", "q_norm", "k_norm") where they are not ``<name>.q_proj.weight`` and so on.
 """
 from __future__ import annotations
 
@@ -49,7 +52,8 @@ class PagedAttention(Mixer):
                  position: PartSpec, bias: bool = True, window: Optional[int] = None,
                  scale: Optional[float] = None, init_std: float = 0.02, v_head_dim: Optional[int] = None,
                  keep_first: int = 0, sink: Optional[float] = None, unit_norm_eps: Optional[float] = None,
-                 output_gate: bool = False, value_mix: Optional[str] = None, tensors: Optional[Mapping[str, str]] = None):
+                 output_gate=False, value_mix: Optional[str] = None, tensors: Optional[Mapping[str, str]] = None,
+                 qk_norm_eps: Optional[float] = None):
         """``v_head_dim``: the width of a value head where it differs from ``head_dim`` (such a layer runs on the
         kernels that take both widths: the plain attention kernel and the unfused projection path)."""
         if n_heads % n_kv_heads:
@@ -63,17 +67,31 @@ class PagedAttention(Mixer):
         self.keep_first = max(int(keep_first or 0), 0) if self.window else 0
         self.sink = None if sink is None else float(sink)
         self.unit_norm_eps = None if unit_norm_eps is None else float(unit_norm_eps)
+        if output_gate not in (False, True, None, "head", "elementwise"):
+            raise ValueError(f"{name}: output_gate '{output_gate}' unknown (False, True or 'elementwise')")
         self.output_gate = bool(output_gate)
+        self.gate_elementwise = output_gate == "elementwise"
+        self.qk_norm_eps = None if qk_norm_eps is None else float(qk_norm_eps)
+        self.q_norm_w = self.k_norm_w = None
         if value_mix not in (None, "source", "mix"):
             raise ValueError(f"{name}: value_mix '{value_mix}' unknown (None, 'source' or 'mix')")
         self.value_mix, self.mix_weight = value_mix, 0.0
         self.names = {"q": f"{name}.q_proj.weight", "k": f"{name}.k_proj.weight", "v": f"{name}.v_proj.weight",
                       "o": f"{name}.o_proj.weight", "q_bias": f"{name}.q_proj.bias", "k_bias": f"{name}.k_proj.bias",
-                      "v_bias": f"{name}.v_proj.bias", "gate": f"{name}.gate.weight", "mix": f"{name}.value_mix"}
+                      "v_bias": f"{name}.v_proj.bias", "gate": f"{name}.gate.weight", "mix": f"{name}.value_mix",
+                      "q_norm": f"{name}.q_norm.weight", "k_norm": f"{name}.k_norm.weight"}
         self.names.update(tensors or {})
         # (what the kernels fused for the plain case do not do: then the projection, the row kernel and attention run one by one)
-        self._extras = self.unit_norm_eps is not None or self.output_gate or self.value_mix is not None
+        self._extras = (self.unit_norm_eps is not None or self.output_gate or self.value_mix is not None
+                        or self.qk_norm_eps is not None)
         self.w_qkv = self.b_qkv = self.w_o = self._w_q = None
+
+    @property
+    def gate_rows(self) -> int:
+        """Rows of the gate's weight: one per head, or one per element of the concatenated heads."""
+        if not self.output_gate:
+            return 0
+        return self.n_heads * self.v_head_dim if self.gate_elementwise else self.n_heads
 
     def cache_spec(self) -> CacheSpec:
         return CacheSpec(self.n_kv_heads, self.head_dim, self.window,
@@ -93,7 +111,10 @@ class PagedAttention(Mixer):
             out[nm["k_bias"]] = ParamSpec((self.n_kv_heads * d,), s)
             out[nm["v_bias"]] = ParamSpec((self.n_kv_heads * dv,), s)
         if self.output_gate:
-            out[nm["gate"]] = ParamSpec((self.n_heads, H), s)
+            out[nm["gate"]] = ParamSpec((self.gate_rows, H), s)
+        if self.qk_norm_eps is not None:
+            out[nm["q_norm"]] = ParamSpec((d,), ("ones",))
+            out[nm["k_norm"]] = ParamSpec((d,), ("ones",))
         if self.value_mix is not None:       # (the source layer's tensor is in the file too, where the file has it; nothing reads it)
             out[nm["mix"]] = ParamSpec((), ("uniform", 0.2, 0.8), optional=self.value_mix == "source")
         return out
@@ -106,11 +127,15 @@ class PagedAttention(Mixer):
         if self.bias:
             biases = [tensors[nm[p + "_bias"]] for p in "qkv"]
             if self.output_gate:
-                biases.append(torch.zeros(self.n_heads, dtype=biases[0].dtype, device=biases[0].device))
+                biases.append(torch.zeros(self.gate_rows, dtype=biases[0].dtype, device=biases[0].device))
             self.b_qkv = concat_weights(biases)
         self.w_o = ops.prepare_linear(tensors[nm["o"]])
         if self.value_mix == "mix":
             self.mix_weight = float(tensors[nm["mix"]].float().item())
+        if self.qk_norm_eps is not None:
+            self.q_norm_w, self.k_norm_w = tensors[nm["q_norm"]], tensors[nm["k_norm"]]
+            if self.q_norm_w.dtype != self.k_norm_w.dtype:
+                self.q_norm_w, self.k_norm_w = self.q_norm_w.float(), self.k_norm_w.float()
         self._w_q = None
 
     def _prepare_qkv(self, weight: torch.Tensor, heads: int):
@@ -148,7 +173,9 @@ class PagedAttention(Mixer):
         t = ctx.timer
         qkv = ops.linear(h, self.w_qkv, keep_slices=True)
         dtype = qkv.dtype
-        gate = torch.empty((T, nH), dtype=torch.float32, device=ctx.device) if self.output_gate else None
+        per_head_gate = self.output_gate and not self.gate_elementwise
+        gate = torch.empty((T, nH), dtype=torch.float32, device=ctx.device) if per_head_gate else None
+        qk_norm = (self.q_norm_w, self.k_norm_w, self.qk_norm_eps) if self.qk_norm_eps is not None else None
         key = ("value_mix", nKV, dv)
         v_first = v_out = None
         if self.value_mix == "source":
@@ -159,10 +186,13 @@ class PagedAttention(Mixer):
             if v_first is None:
                 raise ValueError(f"{self.name}: mixes in the values of an earlier layer, but none has handed any on in this step")
         q = ops.rope_append(qkv, self.b_qkv, ctx.write_slots(cache.group), cos, sin, style, rotary_dim, nH, nKV, d, cache.k, cache.v,
-                            cache.page_size, dv, self.unit_norm_eps, gate, v_first, self.mix_weight, v_out)
+                            cache.page_size, dv, self.unit_norm_eps, gate, v_first, self.mix_weight, v_out, qk_norm,
+                            self.gate_rows if self.gate_elementwise else 0)
         if t is not None:
             t.mark("mixer.qkv")
         a = self._attend(q, cache, ctx, gate)
+        if self.gate_elementwise:         # the gate's columns lie behind q, k and v in the projected rows
+            a = ops.sigmoid_gate(a, qkv, (nH + nKV) * d + nKV * dv)
         if t is not None:
             t.mark("mixer.attention")
         return self._project_out(a, sink)

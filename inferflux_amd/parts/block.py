@@ -14,6 +14,14 @@ x <- x + norm2(ffn(x)); the sub-blocks read the stream itself (rounded to the ac
 have no feed-forward.  Its norms are parts with ``add_to(stream, delta, cast_dtype)``, which adds the normed delta
 into the stream and returns the rounding that the next sub-block reads, all in one kernel.
 
+"hyper" replaces the one stream by ``streams`` copies x_1 .. x_S (all equal to the embedding at the start).  Sub-block q
+(1: the mixer, 2: the feed-forward) with its weights in_q [S], out_q [S], mix_q [S, S] reads u = sum_s in_q[s] x_s, computes
+y = sub-block(norm(u)), and then all streams change at once from the old ones, x_t <- sum_s mix_q[s, t] x_s + out_q[t] y.
+The update is not done where y is made: y travels on as ``HyperPending`` and the kernel that reads the streams for the
+next sub-block (of this layer or the next) updates them first, so a sub-block costs one such kernel.  After the last layer
+the model asks the block to ``close_stream``: the pending update, then the sum of the streams as the one stream that the
+final norm reads.
+
 For steps of few rows a sub-block that can do so adds its output to the stream in its last product's
 epilogue and hands on the next norm's rows up to a factor per row (``ScaledRows``), which the sub-block
 after it applies to its first product's sums: the norm between them then needs no kernel.  Parts that
@@ -26,7 +34,7 @@ import torch
 from ..kernels import ops
 from ..kernels.ops import ScaledDelta, ScaledRows
 from .base import Block, MixerBinding, StreamSink, build_part, register_part
-from .plan import LayerSpec
+from .plan import LayerSpec, ParamSpec
 
 
 def normed_for(norm, reader, residual, pending, ctx):
@@ -164,3 +172,111 @@ class StreamRows:
 
     def __init__(self, stream, rows):
         self.stream, self.rows = stream, rows
+
+
+class HyperStreams:
+    """The S residual streams of a step's rows, float32 [T, S, H], as a "hyper" block hands them to the next."""
+    __slots__ = ("data",)
+
+    def __init__(self, data):
+        self.data = data
+
+    @property
+    def device(self):
+        return self.data.device
+
+
+class HyperPending:
+    """A sub-block's output y that has not changed the streams yet, with the weights that say how it will:
+    x_t <- sum_s mix[s, t] x_s + out[t] y."""
+    __slots__ = ("y", "mix", "out")
+
+    def __init__(self, y, mix, out):
+        self.y, self.mix, self.out = y, mix, out
+
+
+@register_part("block", "hyper")
+class HyperConnectionBlock(Block):
+    """Pre-norm sub-blocks over ``streams`` residual streams (see the module's text).  Tensors: ``<prefix>.hc1.in`` [S],
+    ``.hc1.out`` [S], ``.hc1.mix`` [S, S] (indexed [from, to]) for the mixer and ``.hc2.*`` for the feed-forward; they are
+    widened to float at load."""
+    graph_safe = True
+
+    def __init__(self, layer: LayerSpec, hidden_size: int, streams: int):
+        if layer.norm_in is None or layer.extra or (layer.ffn is None) != (layer.norm_post is None):
+            raise ValueError(f"layer {layer.prefix}: the hyper block is a norm and a mixer, optionally a second norm with a feed-forward")
+        self.prefix, self.hidden_size, self.streams = layer.prefix, int(hidden_size), int(streams)
+        if not 0 < self.streams <= ops.HYPER_MAX_STREAMS:
+            raise ValueError(f"layer {layer.prefix}: {streams} streams (1 to {ops.HYPER_MAX_STREAMS})")
+        self.norm_in = build_part("norm", layer.norm_in, hidden_size=hidden_size)
+        self.mixer = build_part("mixer", layer.mixer, hidden_size=hidden_size)
+        self.norm_post = build_part("norm", layer.norm_post, hidden_size=hidden_size) if layer.norm_post is not None else None
+        self.ffn = build_part("ffn", layer.ffn, hidden_size=hidden_size) if layer.ffn is not None else None
+        for n in (self.norm_in, self.norm_post):
+            if n is not None and n.rms_params() is None and not hasattr(n, "weight"):
+                raise ValueError(f"layer {layer.prefix}: the hyper block reads the streams through RMS norms")
+        self.w = {}
+
+    def children(self):
+        return tuple(p for p in (self.norm_in, self.mixer, self.norm_post, self.ffn) if p is not None)
+
+    def _subs(self):
+        return ("hc1", "hc2") if self.ffn is not None else ("hc1",)
+
+    def param_specs(self):
+        S, out = self.streams, {}
+        for q in self._subs():
+            out[f"{self.prefix}.{q}.in"] = ParamSpec((S,), ("uniform", 0.1, 0.5))
+            out[f"{self.prefix}.{q}.out"] = ParamSpec((S,), ("uniform", 0.5, 1.0))
+            out[f"{self.prefix}.{q}.mix"] = ParamSpec((S, S), ("uniform", 0.0, 0.6))
+        return out
+
+    def load(self, tensors):
+        for q in self._subs():
+            for k in ("in", "out", "mix"):
+                self.w[q, k] = tensors[f"{self.prefix}.{q}.{k}"].float().contiguous()
+        self.ones = torch.ones(self.streams, dtype=torch.float32, device=self.w["hc1", "in"].device)
+
+    def _read(self, streams, pending, sub, norm, ctx):
+        """The streams after the pending update, and what sub-block ``sub`` reads from them through ``norm``."""
+        weight, eps = norm.rms_params()
+        src = streams.data if isinstance(streams, HyperStreams) else streams          # (one stream from the embedding: S copies)
+        y = mix = out = None
+        if isinstance(pending, HyperPending):
+            y, mix, out = pending.y, pending.mix, pending.out
+        elif pending is not None and not getattr(pending, "in_stream", False):
+            raise ValueError(f"layer {self.prefix}: the hyper block was handed a delta of another arrangement")
+        data, rows = ops.hyper_step(src, self.streams, y, mix, out, self.w[sub, "in"], weight, eps, ctx.act_dtype)
+        return HyperStreams(data), rows
+
+    def forward(self, residual, pending, ctx, binding: MixerBinding, following=None):
+        t = ctx.timer
+        if t is not None:
+            t.enter("norm")
+        streams, h = self._read(residual, pending, "hc1", self.norm_in, ctx)
+        if t is not None:
+            t.mark("norm"); t.enter("mixer")
+        pending = HyperPending(self.mixer.forward(h, ctx, binding), self.w["hc1", "mix"], self.w["hc1", "out"])
+        if t is not None:
+            t.mark("mixer")
+        if self.ffn is None:
+            return streams, pending
+        if t is not None:
+            t.enter("norm")
+        streams, h = self._read(streams, pending, "hc2", self.norm_post, ctx)
+        if t is not None:
+            t.mark("norm"); t.enter("ffn")
+        pending = HyperPending(self.ffn.forward(h, ctx), self.w["hc2", "mix"], self.w["hc2", "out"])
+        if t is not None:
+            t.mark("ffn")
+        return streams, pending
+
+    def close_stream(self, residual, pending, ctx):
+        """The one stream the final norm reads: the pending update, then the sum of the streams."""
+        if not isinstance(residual, HyperStreams):
+            return residual, pending
+        y = mix = out = None
+        if isinstance(pending, HyperPending):
+            y, mix, out = pending.y, pending.mix, pending.out
+        _, total = ops.hyper_step(residual.data, self.streams, y, mix, out, self.ones)
+        return total, None

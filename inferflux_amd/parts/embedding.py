@@ -57,8 +57,10 @@ class LinearHead(Part):
     """``tied_to`` names the tensor (the embedding table) a tied head shares; None for its own."""
 
     def __init__(self, name: str, vocab_size: int, hidden_size: int, tied_to: Optional[str] = None, init_std: float = 0.02,
-                 tensor: Optional[str] = None):
-        """``tensor``: the weight's full name in the model file where that is not ``<name>.weight``."""
+                 tensor: Optional[str] = None, scale: float = 1.0, softcap: Optional[float] = None):
+        """``tensor``: the weight's full name in the model file where that is not ``<name>.weight``.  ``scale``: a factor on
+        the logits; ``softcap`` c: after it the logits become c * tanh(logit / c)."""
+        self.scale, self.softcap = float(scale), (float(softcap) if softcap else 0.0)
         self.name, self.vocab_size, self.hidden_size, self.tied_to, self.init_std = name, int(vocab_size), int(hidden_size), tied_to, init_std
         self.tensor = tensor or f"{name}.weight"
         self.weight: Optional[ops.LinearWeight] = None
@@ -75,4 +77,7 @@ class LinearHead(Part):
         return ops.takes_scaled_rows(n_rows, self.weight)
 
     def forward(self, h) -> torch.Tensor:
-        return ops.linear(h, self.weight, out_dtype=torch.float32)
+        logits = ops.linear(h, self.weight, out_dtype=torch.float32)
+        if self.scale != 1.0 or self.softcap:
+            ops.scale_softcap(logits, self.scale, self.softcap)
+        return logits

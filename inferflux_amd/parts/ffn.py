@@ -77,3 +77,41 @@ class SwiGLU(FeedForward):
         if sink is not None and ops.adds_into_stream(a.shape[0], self.w_down, sink.norm_weight):
             return ops.linear_into_stream(a, self.w_down, sink.stream, sink.norm_weight, sink.eps, sink.mult)
         return ops.linear(a, self.w_down, keep_slices=sink is not None)   # an RMS norm's kernel adds partial sums itself
+
+
+@register_part("ffn", "dense_ffn")
+class DenseFFN(FeedForward):
+    """A feed-forward without a gate: down( act(up(x)) ), no biases; act is "gelu_tanh" (the default) or "silu", formed in
+    float.  ``tensors``: the full names of "up" and "down" where they are not ``<name>.up_proj.weight`` and so on."""
+    graph_safe = True
+    adds_to_stream = True
+
+    def __init__(self, name: str, hidden_size: int, intermediate_size: int, init_std: float = 0.02,
+                 activation: str = "gelu_tanh", tensors: Optional[Mapping[str, str]] = None):
+        self.name, self.hidden_size, self.intermediate_size = name, int(hidden_size), int(intermediate_size)
+        self.init_std = init_std
+        if activation not in ACTIVATIONS:
+            raise ValueError(f"{name}: activation '{activation}' unknown (one of {sorted(ACTIVATIONS)})")
+        self.activation, self.act = activation, ACTIVATIONS[activation]
+        self.names = {k: f"{name}.{k}_proj.weight" for k in ("up", "down")}
+        self.names.update(tensors or {})
+        self.w_up = self.w_down = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        H, I, s = self.hidden_size, self.intermediate_size, ("normal", self.init_std)
+        return {self.names["up"]: ParamSpec((I, H), s), self.names["down"]: ParamSpec((H, I), s)}
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        self.w_up = ops.prepare_linear(tensors[self.names["up"]])
+        self.w_down = ops.prepare_linear(tensors[self.names["down"]])
+
+    def accepts_scaled_rows(self, n_rows: int) -> bool:
+        return ops.takes_scaled_rows(n_rows, self.w_up)
+
+    def forward(self, h, ctx, sink=None):
+        a = ops.linear_act(h, self.w_up, self.act)
+        if ctx.timer is not None:
+            ctx.timer.mark("ffn.up")
+        if sink is not None and ops.adds_into_stream(a.shape[0], self.w_down, sink.norm_weight):
+            return ops.linear_into_stream(a, self.w_down, sink.stream, sink.norm_weight, sink.eps, sink.mult)
+        return ops.linear(a, self.w_down, keep_slices=sink is not None)

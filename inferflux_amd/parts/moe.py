@@ -6,8 +6,13 @@
     out = sum over the chosen e of w_e * W_down[e] (silu(W_gate[e] h) * (W_up[e] h)),
     w_e = s_e, divided by the sum of the chosen s with ``renormalize``, times ``route_scale``
 
-Tensors (``<name>.``): router [experts, H], e<j>.gate and e<j>.up [ff, H], e<j>.down [H, ff]; no biases.  The experts'
-matrices are stacked at load into [experts, ff, H] and [experts, H, ff].
+With ``router_bias`` a bias b_r joins the logits, z = W_r h + b_r (it counts for the choice and for the weights).  Scoring
+"softmax" with ``renormalize`` is the softmax over the chosen logits alone.  With ``shared_ff`` a further gated feed-forward
+of that inner size runs for every row and is added, times sigmoid(w_sg . h) (one number per row) with ``shared_gate``.
+
+Tensors (``<name>.``): router [experts, H] (router.b [experts]), e<j>.gate and e<j>.up [ff, H], e<j>.down [H, ff]; shared.gate,
+shared.up, shared.down, shared.sg [1, H]; no other biases.  The experts' matrices are stacked at load into [experts, ff, H]
+and [experts, H, ff].
 
 The router and the choice run on the device, and the experts' products read each (row, choice)'s expert from device
 memory: the launches of a step depend on its layout alone, so a decode step is captured and replayed like any other.
@@ -20,6 +25,7 @@ import torch
 
 from ..kernels import ops
 from .base import FeedForward, register_part
+from .ffn import SwiGLU
 from .plan import ParamSpec
 
 
@@ -34,7 +40,7 @@ class MixtureOfExperts(FeedForward):
 
     def __init__(self, name: str, hidden_size: int, n_experts: int, top: int, ff: int, groups: int = 1, keep_groups: int = 1,
                  group_top: int = 2, scoring: str = "sigmoid", renormalize: bool = False, route_scale: float = 1.0,
-                 init_std: float = 0.02):
+                 init_std: float = 0.02, router_bias: bool = False, shared_ff: int = 0, shared_gate: bool = False):
         if scoring not in ("sigmoid", "softmax"):
             raise ValueError(f"{name}: scoring '{scoring}' unknown (sigmoid or softmax)")
         if n_experts % groups or not 0 < keep_groups <= groups or not 0 < top <= keep_groups * (n_experts // groups):
@@ -44,6 +50,18 @@ class MixtureOfExperts(FeedForward):
         self.groups, self.keep_groups, self.group_top = int(groups), int(keep_groups), int(group_top)
         self.scoring, self.renormalize, self.route_scale, self.init_std = scoring, bool(renormalize), float(route_scale), init_std
         self.router = self.gate = self.up = self.down = None
+        self.router_bias, self.bias = bool(router_bias), None
+        self.shared_gate, self.shared_gate_w = bool(shared_gate), None
+        self.shared = None
+        if shared_ff:
+            n = f"{name}.shared"
+            self.shared = SwiGLU(n, hidden_size, int(shared_ff), init_std, "silu",
+                                 {"gate": f"{n}.gate", "up": f"{n}.up", "down": f"{n}.down"})
+        elif shared_gate:
+            raise ValueError(f"{name}: a gate on a shared expert that does not exist")
+
+    def children(self):
+        return (self.shared,) if self.shared is not None else ()
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         n, H, s = self.name, self.hidden_size, ("normal", self.init_std)
@@ -52,6 +70,10 @@ class MixtureOfExperts(FeedForward):
             out[f"{n}.e{e}.gate"] = ParamSpec((self.ff, H), s)
             out[f"{n}.e{e}.up"] = ParamSpec((self.ff, H), s)
             out[f"{n}.e{e}.down"] = ParamSpec((H, self.ff), s)
+        if self.router_bias:
+            out[f"{n}.router.b"] = ParamSpec((self.n_experts,), s)
+        if self.shared_gate:
+            out[f"{n}.shared.sg"] = ParamSpec((1, H), s)
         return out
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
@@ -65,9 +87,25 @@ class MixtureOfExperts(FeedForward):
             # one tensor that both products read: rows of gate and up in turns of 16
             self.gate, self.up = ops.pair_gate_up(self.gate, self.up), None
 
+        if self.router_bias:
+            self.bias = tensors[f"{n}.router.b"].float().contiguous()        # the router is float whatever the file holds
+        if self.shared_gate:
+            self.shared_gate_w = tensors[f"{n}.shared.sg"].to(dtype).reshape(-1).contiguous()
+
     def route(self, h):
         return ops.moe_route(h, self.router, self.top, self.groups, self.keep_groups, self.group_top,
-                             self.scoring == "softmax", self.renormalize, self.route_scale)
+                             self.scoring == "softmax", self.renormalize, self.route_scale, self.bias)
+
+    def _with_shared(self, out, x, ctx):
+        """The chosen experts' sum plus the shared expert's output (times its gate of one number per row)."""
+        if self.shared is None:
+            return out
+        extra = self.shared.forward(x, ctx)
+        if self.shared_gate:
+            return ops.gated_add(out, extra, x, self.shared_gate_w)
+        a = out.sum(torch.float32) if isinstance(out, ops.SliceSums) else out.float()
+        b = extra.sum(torch.float32) if isinstance(extra, ops.SliceSums) else extra.float()
+        return (a + b).to(x.dtype)
 
     def forward(self, h, ctx):
         x = h if h.dtype == self.router.dtype else h.to(self.router.dtype)
@@ -75,6 +113,6 @@ class MixtureOfExperts(FeedForward):
         if ctx.timer is not None:
             ctx.timer.mark("ffn.route")
         if self.up is None and x.shape[0] * self.top >= GROUPED_MIN_ITEMS:
-            return ops.moe_experts_grouped(x, self.gate, self.down, ids, weights)      # (partial sums, one per choice)
-        out = ops.moe_experts(x, self.gate, self.up, self.down, ids, weights)
+            return self._with_shared(ops.moe_experts_grouped(x, self.gate, self.down, ids, weights), x, ctx)      # (partial sums, one per choice)
+        out = self._with_shared(ops.moe_experts(x, self.gate, self.up, self.down, ids, weights), x, ctx)
         return out if out.dtype == h.dtype else out.to(h.dtype)

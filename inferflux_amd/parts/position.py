@@ -18,6 +18,10 @@ slow): with dim(t) = dims ln(original / (2 pi t)) / (2 ln theta), lo = max(floor
 dims - 1) and ramp_p = clamp((p - lo) / max(hi - lo, 0.001), 0, 1), pair p turns with f_p / factor * ramp_p +
 f_p (1 - ramp_p): the fast pairs keep their frequency, the slow ones are stretched by the factor, and cos and sin are
 both multiplied by 0.1 ln(factor) + 1.
+
+Frequencies scaled in bands of wavelength (``scaling`` = factor, original, low, high): with l_p = 2 pi / f_p, a pair with
+l_p < original / high keeps f_p; one with l_p > original / low turns with f_p / factor; between the two, with
+s = (original / l_p - low) / (high - low), it turns with (1 - s) f_p / factor + s f_p.  cos and sin keep their size.
 """
 from __future__ import annotations
 
@@ -59,7 +63,8 @@ class RotaryPosition(PositionEncoding):
 
     def __init__(self, head_dim: int, theta: float, rotary_dim: Optional[int] = None, style: str = "split_half",
                  scaling: Optional[dict] = None):
-        """``scaling``: None, or {"factor", "original", "fast", "slow"} (see the module's text)."""
+        """``scaling``: None, {"factor", "original", "fast", "slow"} (a ramp over the pairs) or {"factor", "original", "low",
+        "high"} (bands of wavelength); see the module's text."""
         self.head_dim = int(head_dim)
         self.rotary_dim = int(rotary_dim) if rotary_dim is not None else self.head_dim
         self.theta = float(theta)
@@ -70,7 +75,15 @@ class RotaryPosition(PositionEncoding):
         self.style = style
         self.scaling = None
         self.magnitude = 1.0
-        if scaling:
+        self.bands = bool(scaling) and ("low" in scaling or "high" in scaling)
+        if self.bands:
+            missing = [k for k in ("factor", "original", "low", "high") if k not in scaling]
+            if missing:
+                raise ValueError(f"rotary scaling in bands needs {missing}")
+            self.scaling = {k: float(scaling[k]) for k in ("factor", "original", "low", "high")}
+            if self.scaling["factor"] <= 0 or self.scaling["original"] <= 0 or not 0 < self.scaling["low"] < self.scaling["high"]:
+                raise ValueError(f"rotary scaling: factor and original must be positive and 0 < low < high, got {self.scaling}")
+        elif scaling:
             missing = [k for k in ("factor", "original", "fast", "slow") if k not in scaling]
             if missing:
                 raise ValueError(f"rotary scaling needs {missing}")
@@ -88,6 +101,12 @@ class RotaryPosition(PositionEncoding):
         if self.scaling is None:
             return f
         sc, dims = self.scaling, self.rotary_dim
+        if self.bands:
+            wavelength = 2.0 * math.pi / f
+            s = torch.clamp((sc["original"] / wavelength - sc["low"]) / (sc["high"] - sc["low"]), 0.0, 1.0)
+            blended = (1.0 - s) * f / sc["factor"] + s * f
+            return torch.where(wavelength < sc["original"] / sc["high"], f,
+                               torch.where(wavelength > sc["original"] / sc["low"], f / sc["factor"], blended))
         dim_of = lambda turns: dims * math.log(sc["original"] / (2.0 * math.pi * turns)) / (2.0 * math.log(self.theta))
         lo = max(math.floor(dim_of(sc["fast"])), 0)
         hi = min(math.ceil(dim_of(sc["slow"])), dims - 1)
