@@ -206,3 +206,13 @@ def forward(config, W, tokens, return_layers=False):
     if cap:
         logits = cap * np.tanh(logits / cap)
     return (logits, np.stack(after)) if return_layers else logits
+
+
+def greedy_generate(config, W, prompt, n):
+    """n tokens, each the largest logit after everything before it (the whole sequence anew every time)."""
+    ids, out = list(prompt), []
+    for _ in range(n):
+        tok = int(np.argmax(forward(config, W, ids)[-1]))
+        ids.append(tok)
+        out.append(tok)
+    return out
