@@ -88,6 +88,10 @@ class ModelConfig:
         of the model folder).  Most files name every size: they return themselves."""
         return self
 
+    def open_sizes(self) -> Tuple[str, ...]:
+        """What the config still leaves to the tensors' shapes (names for a message); empty when every size is known."""
+        return ()
+
     def save(self, folder: str) -> None:
         os.makedirs(folder, exist_ok=True)
         with open(os.path.join(folder, "config.json"), "w") as f:

@@ -72,7 +72,7 @@ def load_config(folder: str) -> ModelConfig:
     """The typed config of a model folder.  A config whose file leaves a size to a tensor's shape is completed from the
     headers of the folder's weight files (no tensor is read)."""
     cfg = config_from_dict(read_config_json(folder))
-    if type(cfg).with_tensor_shapes is not ModelConfig.with_tensor_shapes:
+    if cfg.open_sizes():
         from ..weights.safetensors_io import open_model_files
         files = open_model_files(folder)
         try:

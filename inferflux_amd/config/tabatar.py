@@ -297,6 +297,9 @@ class TabatarConfig(ModelConfig):
         lp = self.loop
         return tuple(range(lp.start)) + tuple(range(lp.start, lp.stop)) * lp.times + tuple(range(lp.stop, n))
 
+    def open_sizes(self) -> Tuple[str, ...]:
+        return tuple(f"layers[{i}].mixer.rank" for i, L in enumerate(self.layers) if L.type == "gla" and L.mixer.rank is None)
+
     def with_tensor_shapes(self, shapes: Mapping[str, Tuple[int, ...]]) -> "TabatarConfig":
         """The config with the sizes it leaves open taken from the model file: a gla layer's decay rank is the number of
         rows of its ``l<i>.mix.a1``."""
