@@ -198,7 +198,8 @@ __global__ __launch_bounds__(256) void gla_combine_kernel(CombineArgs a) {
 
 template <typename T, int DP>
 static int launch_gla(const GlaArgs& a, int R, int n_chunks, const int* req_chunk0, hipStream_t s) {
-  const int threads = ((a.dv * a.parts + WAVE - 1) / WAVE) * WAVE;
+  // (the first d threads load the stage's q, k and decays: a head of few values still gets a thread per key channel)
+  const int threads = ((max(a.dv * a.parts, a.d) + WAVE - 1) / WAVE) * WAVE;
   IFX_REQUIRE(threads <= GLA_MAX_THREADS(DP), "gla_scan: %d threads a head with %d channels each (at most %d)", threads, DP, GLA_MAX_THREADS(DP));
   const size_t lds = (size_t)STAGE * (3 * a.d + a.dv) * sizeof(float);
   if (n_chunks == 0) {

@@ -1182,7 +1182,7 @@ def gla_layout(d: int, dv: int) -> Tuple[int, int]:
         parts = 1
         while parts * dp < d:
             parts *= 2
-        if parts <= 64 and dv * parts <= max_threads:
+        if parts <= 64 and max(dv * parts, d) <= max_threads:     # (a thread per key channel loads a stage's q, k and decays)
             return dp, parts
     raise KernelError(f"gla: a head of {d} key channels and {dv} values does not fit a workgroup")
 

@@ -93,12 +93,26 @@ def config(name):
     return copy.deepcopy(CONFIGS[name])
 
 
-def write_model(folder, cfg, seed, gain=1.0, keep_rank=False):
+def router_values(n):
+    """n distinct router logits between -2 and 2.6, unevenly spaced, no two closer than half the mean spacing."""
+    import math
+    step = 4.6 / max(n - 1, 1)
+    return [-2.0 + step * k + 0.2 * step * math.sin(1.7 * k + 0.3) for k in range(n)]
+
+
+def write_model(folder, cfg, seed, gain=1.0, keep_rank=False, decisive_router=False):
     """config.json and model.safetensors with seeded weights, bfloat16-representable, shaped so that faults show: norm
     weights away from 1, query/key projections with a gain (peaked attention), decays over the range a trained recurrence
     has (from forgetting within a few tokens to remembering hundreds), router and gate biases that matter, stream
     connections that are neither the identity nor symmetric.  Without ``keep_rank`` the written config.json leaves the
-    recurrences' decay rank to the tensors' shapes."""
+    recurrences' decay rank to the tensors' shapes.
+
+    With ``decisive_router`` no choice of experts is a close call, so that an engine that rounds its activations to
+    bfloat16 makes the choices of the exact model (a choice that rounding flips changes a row's logits altogether and says
+    nothing about the kernels): expert e's router row reads channel e of its input alone, a token's embedding holds a
+    permutation of ``router_values`` on those channels, nothing writes into them (the rows of every matrix that writes into
+    the stream are zero there), the norms before the experts have weight 1 on them and the routers have no bias, so a
+    router's logits are a token's values times one positive number.  (Routers with random weights and biases run in 32-bit.)"""
     from safetensors.torch import save_file
     from inferflux_amd.config import config_from_dict
     from inferflux_amd.engine.model import Model
@@ -128,6 +142,21 @@ def write_model(folder, cfg, seed, gain=1.0, keep_rank=False):
             elif name == "embed":
                 t = t * shape[-1] ** 0.5
         tensors[name] = t.to(torch.bfloat16).contiguous()
+    n = max([L["mlp"]["router"]["experts"] for L in cfg["layers"] if L["mlp"] is not None and L["mlp"]["kind"] == "moe"], default=0)
+    if decisive_router and n:
+        values = torch.tensor(router_values(n))
+        for tok in range(cfg["vocab"]):
+            tensors["embed"][tok, :n] = values[torch.randperm(n, generator=g)].to(torch.bfloat16)
+        for name, t in tensors.items():
+            if name.endswith((".o", ".down")):
+                t[:n] = 0
+            elif name.endswith(".norm2"):
+                t[:n] = 1
+            elif name.endswith(".router"):
+                t.zero_()
+                t[:, :t.shape[0]] = torch.eye(t.shape[0]).to(t.dtype)
+            elif name.endswith(".router.b"):
+                t.zero_()
     os.makedirs(folder, exist_ok=True)
     written = copy.deepcopy(cfg)
     if not keep_rank:
