@@ -95,6 +95,39 @@ PODURAX_SIZES = {
     "medium-attention": (_podurax_shape(2048, 8, 16, 2, 128, 2048, 5632, 4096, 16, 128, "a"), _dense_twin(2048, 8, 16, 128, 2, 5632, 2048)),
     "medium-recurrent": (_podurax_shape(2048, 8, 16, 2, 128, 2048, 5632, 4096, 16, 128, "m"), _dense_twin(2048, 8, 16, 128, 2, 5632, 2048)),
 }
+# Layer sizes for the comparison of the Tabatar design (gated linear attention with a matrix state per head; attention with
+# normed heads and an elementwise gate; hyper-connections over several residual streams; a feed-forward without a gate or a
+# mixture of experts with a gated shared expert) with the framework's closest model, the Podurax design, at equal width, depth,
+# heads, window, feed-forward work (two matrices of 1.5 x the inner size against the gated feed-forward's three) and order of
+# attention and recurrence.  ``pattern``: "a" attention, "g" the recurrence.
+def _tabatar_shape(width, layers, heads, kv_heads, dim, window, ff, g_heads, g_dim, g_vdim, rank, pattern, moe=None, streams=4, vocab=32000):
+    att = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+           "rot": {"base": 5e5, "dims": dim // 2, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 4096}}, "mask": {"size": window}}
+    gla = {"heads": g_heads, "dim": g_dim, "vdim": g_vdim, "tau": 16.0, "rank": rank}
+    mix = {"a": ("attention", att), "g": ("gla", gla)}
+    dense = {"kind": "dense", "ff": ff}
+    mlp = lambda i: dense if moe is None or i % 2 == 0 else {"kind": "moe", "expert": {"ff": moe[2]}, "router": {"experts": moe[0], "top": moe[1]},
+                                                              "shared": {"ff": moe[3]}}
+    return {"architecture": "Tabatar", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0}, "streams": streams,
+            "logit_scale": 1.0, "logit_softcap": 30.0,
+            "layers": [{"type": mix[pattern[i % len(pattern)]][0], "mixer": mix[pattern[i % len(pattern)]][1], "mlp": mlp(i)} for i in range(layers)]}
+
+
+TABATAR_SIZES = {
+    "small": (_tabatar_shape(1024, 8, 8, 2, 128, 1024, 4224, 8, 64, 128, 64, "ggag"),
+              _podurax_shape(1024, 8, 8, 2, 128, 1024, 2816, 2048, 16, 64, "mmam")),
+    "medium": (_tabatar_shape(2048, 8, 16, 2, 128, 2048, 8448, 16, 64, 128, 128, "ggag"),
+               _podurax_shape(2048, 8, 16, 2, 128, 2048, 5632, 4096, 16, 128, "mmam")),
+    "medium-attention": (_tabatar_shape(2048, 8, 16, 2, 128, 2048, 8448, 16, 64, 128, 128, "a"),
+                         _podurax_shape(2048, 8, 16, 2, 128, 2048, 5632, 4096, 16, 128, "a")),
+    "medium-recurrent": (_tabatar_shape(2048, 8, 16, 2, 128, 2048, 8448, 16, 64, 128, 128, "g"),
+                         _podurax_shape(2048, 8, 16, 2, 128, 2048, 5632, 4096, 16, 128, "m")),
+    # every second layer a mixture of 32 experts of which a token takes 4, and a shared expert: 4 x 1,760 + 1,408 = 8,448 inner rows a token
+    "medium-experts": (_tabatar_shape(2048, 8, 16, 2, 128, 2048, 8448, 16, 64, 128, 128, "ggag", moe=(32, 4, 1760, 1408)),
+                       _podurax_shape(2048, 8, 16, 2, 128, 2048, 5632, 4096, 16, 128, "mmam")),
+    "medium-one-stream": (_tabatar_shape(2048, 8, 16, 2, 128, 2048, 8448, 16, 64, 128, 128, "ggag", streams=None),
+                          _podurax_shape(2048, 8, 16, 2, 128, 2048, 5632, 4096, 16, 128, "mmam")),
+}
 CONTEXT = 4096
 PROMPT = 2048
 DECODE_KV_START = 3072      # mean context of a 2,048-token decode after a 2,048-token prompt
@@ -118,14 +151,15 @@ def main() -> int:
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--no-gemm-tuning", action="store_true", help="leave the library's default kernel choice for large products")
-    ap.add_argument("--workload", choices=["decode", "prefill", "mumusun", "podurax", *WORKLOADS], default="decode",
+    ap.add_argument("--workload", choices=["decode", "prefill", "mumusun", "podurax", "tabatar", *WORKLOADS], default="decode",
                     help="decode: the headline measurement; prefill: only the 2,048-token prefill, --steps times "
                          "(for profiles); mixed3b / long14b: whole workloads through the scheduler; mumusun: prefill and "
-                         "decode of the Mumusun design beside the dense decoder at equal size (--size, --only-design)")
-    ap.add_argument("--size", choices=["all", *dict.fromkeys([*DESIGN_SIZES, *PODURAX_SIZES])], default="all",
-                    help="--workload mumusun / podurax: which of its sizes")
-    ap.add_argument("--only-design", choices=["both", "mumusun", "podurax", "dense"], default="both",
-                    help="--workload mumusun / podurax: which of the two models")
+                         "decode of the Mumusun design beside the dense decoder at equal size (--size, --only-design); podurax: the same "
+                         "for the Podurax design; tabatar: the Tabatar design beside the Podurax design at equal size")
+    ap.add_argument("--size", choices=["all", *dict.fromkeys([*DESIGN_SIZES, *PODURAX_SIZES, *TABATAR_SIZES])], default="all",
+                    help="--workload mumusun / podurax / tabatar: which of its sizes")
+    ap.add_argument("--only-design", choices=["both", "mumusun", "podurax", "tabatar", "dense"], default="both",
+                    help="--workload mumusun / podurax / tabatar: which of the two models")
     ap.add_argument("--no-decode-weight-copy", action="store_true",
                     help="decode from the weights' plain rows instead of the tiled copy")
     ap.add_argument("--ceilings", action=argparse.BooleanOptionalAction, default=True,
@@ -164,6 +198,8 @@ def main() -> int:
         return run_workload(args, WORKLOADS[args.workload])
     if args.workload == "podurax":
         return run_design_compare(args, PODURAX_SIZES, "podurax")
+    if args.workload == "tabatar":
+        return run_design_compare(args, TABATAR_SIZES, "tabatar", twin="podurax")
     if args.workload == "mumusun":
         return run_design_compare(args)
     shape = dict({"7b": SHAPE_7B, "3b": SHAPE_3B, "14b": SHAPE_14B, "1.5b": SHAPE_15B, "0.5b": SHAPE_05B, "32b": SHAPE_32B,
@@ -460,8 +496,8 @@ def run_workload(args, w) -> int:
     return 0
 
 
-def run_design_compare(args, sizes=None, name="mumusun") -> int:
-    """Prefill and decode throughput of a design (``name``, its sizes in ``sizes``) beside the dense decoder at equal size, through the step
+def run_design_compare(args, sizes=None, name="mumusun", twin="dense") -> int:
+    """Prefill and decode throughput of a design (``name``, its sizes in ``sizes``) beside ``twin`` (the dense decoder, or another design) at equal size, through the step
     function (no scheduler, no sampling): a prompt of --prompt-len tokens whole, and decode steps of 1, 8 and 64
     requests that each hold --context tokens.  One JSON line with every number."""
     import torch
@@ -478,7 +514,7 @@ def run_design_compare(args, sizes=None, name="mumusun") -> int:
     for size, shapes in sizes.items():
         if args.size not in ("all", size):
             continue
-        for design, shape in zip((name, "dense"), shapes):
+        for design, shape in zip((name, twin), shapes):
             if args.only_design not in ("both", design):
                 continue
             cfg = config_from_dict(shape)
@@ -525,12 +561,14 @@ def run_design_compare(args, sizes=None, name="mumusun") -> int:
             print(note, file=sys.stderr, flush=True)
             del runner, model
             torch.cuda.empty_cache()
-    first_of_each = lambda layers: list({L["type"]: L for L in layers}.values())      # one layer of every kind the size has
-    print(json.dumps({"metric": f"prefill and decode tokens/s of the {name.capitalize()} design beside the dense decoder at equal size "
+    first_of_each = lambda layers: list({L["type"] + (L["mlp"] or {}).get("kind", ""): L for L in layers}.values())      # one layer of every kind the size has
+    twin_sizes = lambda shape: first_of_each(shape["layers"]) if "layers" in shape else {
+        kk: shape[kk] for kk in ("hidden_size", "num_attention_heads", "num_key_value_heads", "head_dim", "intermediate_size", "sliding_window")}
+    beside = "the dense decoder" if twin == "dense" else f"the {twin.capitalize()} design"
+    print(json.dumps({"metric": f"prefill and decode tokens/s of the {name.capitalize()} design beside {beside} at equal size "
                                 f"({args.dtype}, random weights, {len(sizes['small'][0]['layers'])} layers each)",
-                      "dtype": args.dtype, "data": "synthetic", "sizes": {k: {name: first_of_each(v[0]["layers"]), "dense": {
-                          kk: v[1][kk] for kk in ("hidden_size", "num_attention_heads", "num_key_value_heads", "head_dim", "intermediate_size", "sliding_window")}}
-                          for k, v in sizes.items() if args.size in ("all", k)},
+                      "dtype": args.dtype, "data": "synthetic", "sizes": {k: {name: first_of_each(v[0]["layers"]), twin: twin_sizes(v[1])}
+                                                                          for k, v in sizes.items() if args.size in ("all", k)},
                       "results": results}), flush=True)
     return 0
 

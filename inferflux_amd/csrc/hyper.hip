@@ -102,6 +102,107 @@ __global__ __launch_bounds__(256) void hc_kernel(HcArgs a) {
   }
 }
 
+// The same for rows whose width is a multiple of 4: a thread takes 4 neighbouring columns a trip, in 16-byte pieces (8-byte ones
+// for y in bfloat16), and asks for everything a trip reads before it uses any of it: steps of few rows are a chain of
+// trips to memory otherwise.  (A stream's element is read and written by the same thread, so updating in place is safe.)
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 hc_bf16x4;
+
+template <int S_MAX>
+__global__ __launch_bounds__(256) void hc_vec_kernel(HcArgs a) {
+  extern __shared__ float u_row[];       // [H]
+  __shared__ float red[16];
+  __shared__ float w_mix[MAX_STREAMS * MAX_STREAMS], w_out[MAX_STREAMS], w_in[MAX_STREAMS];
+  const int S = a.S, H = a.H;
+  const size_t t = blockIdx.x;
+  if (threadIdx.x < S * S && a.y) w_mix[threadIdx.x] = a.mix[threadIdx.x];
+  if (threadIdx.x < S) {
+    w_out[threadIdx.x] = a.y ? a.outw[threadIdx.x] : 0.f;
+    w_in[threadIdx.x] = a.inw ? a.inw[threadIdx.x] : 0.f;
+  }
+  __syncthreads();
+  const float* src = a.src + (a.broadcast ? t * H : t * S * H);
+  float* dst = a.dst ? a.dst + t * S * H : nullptr;
+  const bool y_bf16 = a.y && a.n_slices == 1 && a.y_dtype == DT_BF16;
+  float ss = 0.f;
+  for (int c = threadIdx.x * 4; c < H; c += 1024) {
+    float4 x[S_MAX];
+    if (a.broadcast) {
+      const float4 v = *(const float4*)(src + c);
+#pragma unroll
+      for (int s = 0; s < S_MAX; ++s) x[s] = v;
+    } else {
+#pragma unroll
+      for (int s = 0; s < S_MAX; ++s) x[s] = s < S ? *(const float4*)(src + (size_t)s * H + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    if (a.y) {
+      float4 y;
+      if (y_bf16) {
+        const hc_bf16x4 v = *(const hc_bf16x4*)((const bf16_t*)a.y + t * H + c);
+        y = make_float4((float)v[0], (float)v[1], (float)v[2], (float)v[3]);
+      } else {                            // float, or float partial sums added in slice order
+        const float* part = (const float*)a.y + t * H + c;
+        y = *(const float4*)part;
+        for (int k = 1; k < a.n_slices; ++k) {
+          const float4 v = *(const float4*)(part + (size_t)k * a.slice_stride);
+          y.x += v.x; y.y += v.y; y.z += v.z; y.w += v.w;
+        }
+      }
+      y.x *= a.y_scale; y.y *= a.y_scale; y.z *= a.y_scale; y.w *= a.y_scale;
+      float4 n[S_MAX];
+#pragma unroll
+      for (int to = 0; to < S_MAX; ++to) {
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int s = 0; s < S_MAX; ++s)
+          if (s < S && to < S) {
+            const float m = w_mix[s * S + to];
+            v.x = fmaf(m, x[s].x, v.x); v.y = fmaf(m, x[s].y, v.y); v.z = fmaf(m, x[s].z, v.z); v.w = fmaf(m, x[s].w, v.w);
+          }
+        const float o = w_out[to < S ? to : 0];
+        n[to] = make_float4(fmaf(o, y.x, v.x), fmaf(o, y.y, v.y), fmaf(o, y.z, v.z), fmaf(o, y.w, v.w));
+      }
+#pragma unroll
+      for (int s = 0; s < S_MAX; ++s) x[s] = n[s];
+    }
+    if (dst && (a.y || a.broadcast)) {
+#pragma unroll
+      for (int s = 0; s < S_MAX; ++s)
+        if (s < S) *(float4*)(dst + (size_t)s * H + c) = x[s];
+    }
+    if (a.inw) {
+      float4 u = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int s = 0; s < S_MAX; ++s)
+        if (s < S) {
+          const float w = w_in[s];
+          u.x = fmaf(w, x[s].x, u.x); u.y = fmaf(w, x[s].y, u.y); u.z = fmaf(w, x[s].z, u.z); u.w = fmaf(w, x[s].w, u.w);
+        }
+      *(float4*)(u_row + c) = u;
+      ss = fmaf(u.x, u.x, ss); ss = fmaf(u.y, u.y, ss); ss = fmaf(u.z, u.z, ss); ss = fmaf(u.w, u.w, ss);
+    }
+  }
+  if (!a.inw) return;
+  if (!a.norm_w) {
+    for (int c = threadIdx.x * 4; c < H; c += 1024) *(float4*)((float*)a.out + t * H + c) = *(const float4*)(u_row + c);     // (a thread reads what it wrote)
+    return;
+  }
+  const float inv = rsqrtf(block_sum(ss, red) / (float)H + a.eps);
+  for (int c = threadIdx.x * 4; c < H; c += 1024) {
+    const float4 u = *(const float4*)(u_row + c);
+    float v[4] = {u.x * inv, u.y * inv, u.z * inv, u.w * inv};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] *= load_dyn(a.norm_w, a.norm_dtype, c + e);
+    if (a.out_dtype == DT_F32) {
+      *(float4*)((float*)a.out + t * H + c) = make_float4(v[0], v[1], v[2], v[3]);
+    } else {
+      hc_bf16x4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = (__bf16)v[e];
+      *(hc_bf16x4*)((bf16_t*)a.out + t * H + c) = o;
+    }
+  }
+}
+
 extern "C" int ifx_hyper_step(const float* src, int broadcast, float* dst, const void* y, int y_dtype, int n_slices,
                               long long slice_stride, float y_scale, const float* mix, const float* outw, const float* inw,
                               const void* norm_w, int norm_dtype, float eps, void* out, int out_dtype, int T, int S, int H,
@@ -116,6 +217,17 @@ extern "C" int ifx_hyper_step(const float* src, int broadcast, float* dst, const
   HcArgs a{src, broadcast, dst, y, y_dtype, n_slices, (size_t)slice_stride, y_scale, mix, outw, inw, norm_w, norm_dtype, eps, out, out_dtype, S, H};
   const size_t lds = (size_t)H * sizeof(float);
   hipStream_t s = (hipStream_t)stream;
+  const auto aligned = [](const void* p) { return ((size_t)p & 15) == 0; };
+  const bool y_halves = n_slices == 1 && y_dtype == DT_BF16;
+  const bool vec = H % 4 == 0 && aligned(src) && aligned(dst) && aligned(out) && (n_slices == 1 || slice_stride % 4 == 0) &&
+                   (y_halves ? ((size_t)y & 7) == 0 : aligned(y));
+  if (vec) {
+    if (S <= 1) hipLaunchKernelGGL(hc_vec_kernel<1>, dim3(T), dim3(256), lds, s, a);
+    else if (S <= 2) hipLaunchKernelGGL(hc_vec_kernel<2>, dim3(T), dim3(256), lds, s, a);
+    else if (S <= 4) hipLaunchKernelGGL(hc_vec_kernel<4>, dim3(T), dim3(256), lds, s, a);
+    else hipLaunchKernelGGL(hc_vec_kernel<8>, dim3(T), dim3(256), lds, s, a);
+    IFX_LAUNCH_CHECK();
+  }
   if (S <= 1) hipLaunchKernelGGL(hc_kernel<1>, dim3(T), dim3(256), lds, s, a);
   else if (S <= 2) hipLaunchKernelGGL(hc_kernel<2>, dim3(T), dim3(256), lds, s, a);
   else if (S <= 4) hipLaunchKernelGGL(hc_kernel<4>, dim3(T), dim3(256), lds, s, a);

@@ -1,5 +1,6 @@
 // Small kernels over a step's rows that sit between products:
-//   activation     out = act(x), act the tanh form of gelu or silu (a feed-forward without a gate)
+//   activation     out = act(x), act the tanh form of gelu or silu (a feed-forward without a gate); x may be a product's
+//                  float partial sums
 //   sigmoid_gate   out[t, c] = x[t, c] * sigmoid(g[t, c]), g columns of a wider projected row (or float partial sums of it)
 //   gated_add      out[t, c] = sum_slices base[.][t, c] + sigmoid(h[t] . w) * extra[t, c]: a branch that every row takes,
 //                  weighted by one number per row, added to the sum of the other branches
@@ -43,6 +44,37 @@ extern "C" int ifx_activation(const void* x, void* out, int dtype, long long n, 
   else if (dtype == DT_F32)
     hipLaunchKernelGGL(activation_kernel<float>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (const float*)x, (float*)out, (size_t)n, act);
   else IFX_FAIL("activation: unknown dtype %d", dtype);
+  IFX_LAUNCH_CHECK();
+}
+
+// act of a product left as float partial sums [n_slices][n] (added in slice order), written in the activation type
+template <typename T>
+__global__ __launch_bounds__(256) void activation_slices_kernel(const float* __restrict__ parts, int n_slices, size_t stride,
+                                                                T* __restrict__ out, size_t n4, int act) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n4) return;
+  float4 v = ((const float4*)parts)[i];
+  for (int k = 1; k < n_slices; ++k) {
+    const float4 w = *(const float4*)(parts + (size_t)k * stride + i * 4);
+    v.x += w.x; v.y += w.y; v.z += w.z; v.w += w.w;
+  }
+  const float f[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) out[i * 4 + e] = from_f<T>(act == ACT_GELU_TANH ? act_gelu_tanh(f[e]) : act_silu(f[e]));
+}
+
+extern "C" int ifx_activation_slices(const float* parts, int n_slices, long long stride, void* out, int out_dtype, long long n,
+                                     int act, void* stream) {
+  IFX_REQUIRE(n >= 0 && n % 4 == 0 && stride % 4 == 0 && n_slices >= 1 && (act == ACT_SILU || act == ACT_GELU_TANH),
+              "activation_slices: n=%lld stride=%lld slices=%d act=%d", n, stride, n_slices, act);
+  if (n == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const unsigned blocks = (unsigned)((n / 4 + 255) / 256);
+  if (out_dtype == DT_BF16)
+    hipLaunchKernelGGL(activation_slices_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, parts, n_slices, (size_t)stride, (bf16_t*)out, (size_t)(n / 4), act);
+  else if (out_dtype == DT_F32)
+    hipLaunchKernelGGL(activation_slices_kernel<float>, dim3(blocks), dim3(256), 0, s, parts, n_slices, (size_t)stride, (float*)out, (size_t)(n / 4), act);
+  else IFX_FAIL("activation_slices: unknown dtype %d", out_dtype);
   IFX_LAUNCH_CHECK();
 }
 

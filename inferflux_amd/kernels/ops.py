@@ -743,6 +743,8 @@ def adds_into_stream(n_rows: int, weight, norm_weight: torch.Tensor) -> bool:
     if not isinstance(weight, LinearWeight) or weight.order is not None:
         return False
     N, K = weight.rows.shape
+    if norm_weight is None:           # (a reader that takes partial sums but keeps the addition to itself)
+        return False
     return (weight.rows.dtype == torch.bfloat16 and norm_weight.dtype == torch.bfloat16 and n_rows <= 16 and N % 4 == 0
             and _small_m_kernel(n_rows, N, K, weight.tiled is not None) == "skinny")
 
@@ -1296,11 +1298,22 @@ def hyper_step(src: torch.Tensor, n_streams: int, y=None, mix: Optional[torch.Te
 def linear_act(x, weight, act: int) -> torch.Tensor:
     """act(x W^T) for a feed-forward without a gate (``act``: ACT_SILU or ACT_GELU_TANH, formed in float on the product's
     output)."""
-    return activation(linear(x, weight), act)
+    return activation(linear(x, weight, keep_slices=True), act)
 
 
-def activation(x: torch.Tensor, act: int) -> torch.Tensor:
-    """act(x) element by element in float: ACT_SILU or ACT_GELU_TANH (a feed-forward without a gate)."""
+def activation(x, act: int) -> torch.Tensor:
+    """act(x) element by element in float: ACT_SILU or ACT_GELU_TANH (a feed-forward without a gate).  ``x`` may be
+    ``SliceSums``: the partial sums are added in slice order first, and the result has the type they stand for."""
+    if isinstance(x, SliceSums):
+        parts = x.parts
+        _check(parts, "x", (None, None, None), torch.float32)
+        n = parts.shape[1] * parts.shape[2]
+        if n % 4:
+            return activation(x.sum(x.dtype), act)
+        out = torch.empty(parts.shape[1:], dtype=x.dtype, device=parts.device)
+        _call(load_module("rowwise"), "ifx_activation_slices", (P, I, LL, P, I, LL, I, P), parts.data_ptr(), parts.shape[0], n,
+              out.data_ptr(), _DT[x.dtype], n, int(act), _stream())
+        return out
     _check(x, "x")
     out = torch.empty_like(x)
     _call(load_module("rowwise"), "ifx_activation", (P, P, I, LL, I, P), x.data_ptr(), out.data_ptr(), _dt(x), x.numel(), int(act), _stream())

@@ -132,9 +132,10 @@ class MixerBinding:
 class StreamSink:
     """Where a mixer or feed-forward may add its result itself: the float32 stream, and the weight and eps
     of the RMS norm that reads the stream next.  ``mult`` is the factor on what is added (a model's factor on every
-    sub-block's output; 1 otherwise)."""
-    stream: torch.Tensor
-    norm_weight: torch.Tensor
+    sub-block's output; 1 otherwise).  Without a stream and a norm (both None) nothing may be added, but the reader takes a
+    product left as partial sums (``SliceSums``) and adds them up itself."""
+    stream: Optional[torch.Tensor]
+    norm_weight: Optional[torch.Tensor]
     eps: float
     mult: float = 1.0
 

@@ -195,6 +195,9 @@ class HyperPending:
         self.y, self.mix, self.out = y, mix, out
 
 
+_PARTIAL_SUMS_WELCOME = StreamSink(None, None, 0.0)
+
+
 @register_part("block", "hyper")
 class HyperConnectionBlock(Block):
     """Pre-norm sub-blocks over ``streams`` residual streams (see the module's text).  Tensors: ``<prefix>.hc1.in`` [S],
@@ -249,6 +252,14 @@ class HyperConnectionBlock(Block):
         data, rows = ops.hyper_step(src, self.streams, y, mix, out, self.w[sub, "in"], weight, eps, ctx.act_dtype)
         return HyperStreams(data), rows
 
+    @staticmethod
+    def _run(part, h, ctx, *binding):
+        """A sub-block's output; one that can leave its last product as partial sums is told that the kernel which updates
+        the streams adds them up (nothing is added to a stream where it is made: every stream changes at once)."""
+        if getattr(part, "adds_to_stream", False):
+            return part.forward(h, ctx, *binding, sink=_PARTIAL_SUMS_WELCOME)
+        return part.forward(h, ctx, *binding)
+
     def forward(self, residual, pending, ctx, binding: MixerBinding, following=None):
         t = ctx.timer
         if t is not None:
@@ -256,7 +267,7 @@ class HyperConnectionBlock(Block):
         streams, h = self._read(residual, pending, "hc1", self.norm_in, ctx)
         if t is not None:
             t.mark("norm"); t.enter("mixer")
-        pending = HyperPending(self.mixer.forward(h, ctx, binding), self.w["hc1", "mix"], self.w["hc1", "out"])
+        pending = HyperPending(self._run(self.mixer, h, ctx, binding), self.w["hc1", "mix"], self.w["hc1", "out"])
         if t is not None:
             t.mark("mixer")
         if self.ffn is None:
@@ -266,7 +277,7 @@ class HyperConnectionBlock(Block):
         streams, h = self._read(streams, pending, "hc2", self.norm_post, ctx)
         if t is not None:
             t.mark("norm"); t.enter("ffn")
-        pending = HyperPending(self.ffn.forward(h, ctx), self.w["hc2", "mix"], self.w["hc2", "out"])
+        pending = HyperPending(self._run(self.ffn, h, ctx), self.w["hc2", "mix"], self.w["hc2", "out"])
         if t is not None:
             t.mark("ffn")
         return streams, pending

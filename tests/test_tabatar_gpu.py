@@ -342,7 +342,7 @@ def test_a_key_far_back_is_still_in_the_state(dtype, chunked):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("S", [1, 2, 3, 4, 5, 8])
-@pytest.mark.parametrize("T,H", [(1, 64), (9, 100), (70, 384), (3, 5000)])
+@pytest.mark.parametrize("T,H", [(1, 64), (9, 100), (70, 384), (3, 5000), (5, 99), (2, 2050)])
 def test_hyper_connections_read_and_update_all_streams_at_once(dtype, S, T, H):
     dt, eps = DT[dtype], 1e-5
     g = torch.Generator().manual_seed(S * 100 + T)
@@ -385,6 +385,10 @@ def test_feed_forward_without_a_gate(dtype, M, K, ff):
     x, up = rnd(50, M, K).to(dt), rnd(51, ff, K, scale=2.0 * K ** -0.5).to(dt)
     got = ops.linear_act(x.to(DEV), ops.prepare_linear(up.to(DEV)), ops.ACT_GELU_TANH).cpu()
     assert rel_err(got, T64(pt.gelu_tanh(N64(x) @ N64(up).T))) < (1e-5 if dtype == "float32" else 1.5e-2)
+    pre = N64(x) @ N64(up).T                                        # a product left as partial sums is added up on the way
+    parts = ops.SliceSums(torch.stack([T64(pre * 0.25), T64(pre * 0.5), T64(pre * 0.25)]).float().to(DEV), dt)
+    got = ops.activation(parts, ops.ACT_GELU_TANH)
+    assert got.dtype == dt and rel_err(got.cpu(), T64(pt.gelu_tanh(pre))) < (1e-5 if dtype == "float32" else 6e-3)
     z = torch.linspace(-6, 6, 4001, dtype=torch.float32)
     assert rel_err(ops.activation(z.to(DEV), ops.ACT_GELU_TANH).cpu(), T64(pt.gelu_tanh(N64(z)))) < 1e-6
     assert rel_err(ops.activation(z.to(DEV), ops.ACT_SILU).cpu(), T64(pt.silu(N64(z)))) < 1e-6
