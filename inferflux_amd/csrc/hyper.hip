@@ -108,7 +108,7 @@ __global__ __launch_bounds__(256) void hc_kernel(HcArgs a) {
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 hc_bf16x4;
 
 template <int S_MAX>
-__global__ __launch_bounds__(256) void hc_vec_kernel(HcArgs a) {
+__global__ __launch_bounds__(512) void hc_vec_kernel(HcArgs a) {
   extern __shared__ float u_row[];       // [H]
   __shared__ float red[16];
   __shared__ float w_mix[MAX_STREAMS * MAX_STREAMS], w_out[MAX_STREAMS], w_in[MAX_STREAMS];
@@ -123,8 +123,9 @@ __global__ __launch_bounds__(256) void hc_vec_kernel(HcArgs a) {
   const float* src = a.src + (a.broadcast ? t * H : t * S * H);
   float* dst = a.dst ? a.dst + t * S * H : nullptr;
   const bool y_bf16 = a.y && a.n_slices == 1 && a.y_dtype == DT_BF16;
+  const int stride = blockDim.x * 4;
   float ss = 0.f;
-  for (int c = threadIdx.x * 4; c < H; c += 1024) {
+  for (int c = threadIdx.x * 4; c < H; c += stride) {
     float4 x[S_MAX];
     if (a.broadcast) {
       const float4 v = *(const float4*)(src + c);
@@ -183,11 +184,11 @@ __global__ __launch_bounds__(256) void hc_vec_kernel(HcArgs a) {
   }
   if (!a.inw) return;
   if (!a.norm_w) {
-    for (int c = threadIdx.x * 4; c < H; c += 1024) *(float4*)((float*)a.out + t * H + c) = *(const float4*)(u_row + c);     // (a thread reads what it wrote)
+    for (int c = threadIdx.x * 4; c < H; c += stride) *(float4*)((float*)a.out + t * H + c) = *(const float4*)(u_row + c);     // (a thread reads what it wrote)
     return;
   }
   const float inv = rsqrtf(block_sum(ss, red) / (float)H + a.eps);
-  for (int c = threadIdx.x * 4; c < H; c += 1024) {
+  for (int c = threadIdx.x * 4; c < H; c += stride) {
     const float4 u = *(const float4*)(u_row + c);
     float v[4] = {u.x * inv, u.y * inv, u.z * inv, u.w * inv};
 #pragma unroll
@@ -222,10 +223,12 @@ extern "C" int ifx_hyper_step(const float* src, int broadcast, float* dst, const
   const bool vec = H % 4 == 0 && aligned(src) && aligned(dst) && aligned(out) && (n_slices == 1 || slice_stride % 4 == 0) &&
                    (y_halves ? ((size_t)y & 7) == 0 : aligned(y));
   if (vec) {
-    if (S <= 1) hipLaunchKernelGGL(hc_vec_kernel<1>, dim3(T), dim3(256), lds, s, a);
-    else if (S <= 2) hipLaunchKernelGGL(hc_vec_kernel<2>, dim3(T), dim3(256), lds, s, a);
-    else if (S <= 4) hipLaunchKernelGGL(hc_vec_kernel<4>, dim3(T), dim3(256), lds, s, a);
-    else hipLaunchKernelGGL(hc_vec_kernel<8>, dim3(T), dim3(256), lds, s, a);
+    // (a thread per 4 columns up to 512 threads: a step of few rows has one trip to memory instead of several in a row)
+    const int threads = min(512, ((H / 4 + WAVE - 1) / WAVE) * WAVE);
+    if (S <= 1) hipLaunchKernelGGL(hc_vec_kernel<1>, dim3(T), dim3(threads), lds, s, a);
+    else if (S <= 2) hipLaunchKernelGGL(hc_vec_kernel<2>, dim3(T), dim3(threads), lds, s, a);
+    else if (S <= 4) hipLaunchKernelGGL(hc_vec_kernel<4>, dim3(T), dim3(threads), lds, s, a);
+    else hipLaunchKernelGGL(hc_vec_kernel<8>, dim3(T), dim3(threads), lds, s, a);
     IFX_LAUNCH_CHECK();
   }
   if (S <= 1) hipLaunchKernelGGL(hc_kernel<1>, dim3(T), dim3(256), lds, s, a);
