@@ -11,10 +11,10 @@
 // Decays, their logarithms, S, o, the norm and the gate are float whatever the activation type.
 //
 // A request's S lives in its state slot, one float32 row per slot laid out [head][j][PARTS * DP]: a column j of S as
-// PARTS runs of DP channels (channels at or beyond d are zero and stay zero).  A thread owns one run: DP numbers of S in
-// registers; the PARTS threads of a column are neighbours in a wave and add their parts of o_t[j] by shuffles in a fixed
+// PARTS runs of DP channels (channels at or beyond d are zero and stay zero).  A thread owns one run of one column (of two
+// neighbouring columns where DP <= 32): DP (2 DP) numbers of S in registers; the PARTS threads of a column are neighbours in a wave and add their parts of o_t[j] by shuffles in a fixed
 // order.  A workgroup is one head of one request (or of one chunk): dv * PARTS threads.  Tokens are taken STAGE at a time:
-// the first d threads put q, k and alpha of the stage's tokens into LDS (and form alpha on the way), everybody walks the
+// the threads put q, k and alpha of the stage's tokens into LDS, a (token, channel) each (and form alpha on the way), everybody walks the
 // stage's tokens, o goes to LDS, and a wave per token norms and gates it.
 //
 // MODE 0: a request's rows in one walk, from its slot and back into it.
@@ -59,7 +59,7 @@ __device__ __forceinline__ float log_sigmoid(float x) {      // -softplus(-x), w
 // (a thread's registers hold DP numbers of S: the more of them, the fewer threads a workgroup may have)
 #define GLA_MAX_THREADS(DP) ((DP) <= 32 ? 1024 : ((DP) <= 64 ? 512 : 256))
 
-template <typename T, int DP, int MODE>
+template <typename T, int DP, int MODE, int COLS>
 __global__ __launch_bounds__(GLA_MAX_THREADS(DP)) void gla_kernel(GlaArgs a) {
   extern __shared__ float lds[];
   const int d = a.d, dv = a.dv, parts = a.parts, H = a.H;
@@ -67,6 +67,7 @@ __global__ __launch_bounds__(GLA_MAX_THREADS(DP)) void gla_kernel(GlaArgs a) {
   float* lk = lq + STAGE * d;            // [STAGE][d]
   float* la = lk + STAGE * d;            // [STAGE][d]
   float* lo = la + STAGE * d;            // [STAGE][dv]
+  float* lg = lo + STAGE * dv;           // [STAGE][d]: the decays' logarithms (MODE 1 sums them per channel)
   const int unit = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
   int t0, n;
   size_t s_at;                            // where this head's S lies
@@ -80,66 +81,76 @@ __global__ __launch_bounds__(GLA_MAX_THREADS(DP)) void gla_kernel(GlaArgs a) {
   }
   if (n <= 0) return;
   s_at = (size_t)head * dv * parts * DP;
-  const int j = tid / parts, p = tid % parts;
-  const bool owner = j < dv;
-  float S[DP];
-  float* sp = sbase + s_at + ((size_t)j * parts + p) * DP;
-  if (MODE != 1 && owner) {
+  // a thread owns COLS neighbouring columns j0 .. j0 + COLS - 1 of S for its run of DP channels: what it reads of a token's
+  // q, k and decays from LDS serves COLS columns
+  const int j0 = (tid / parts) * COLS, p = tid % parts;
+  float S[COLS][DP];
+  float* sp = sbase + s_at + ((size_t)j0 * parts + p) * DP;          // (column j0 + c lies c * parts * DP further)
 #pragma unroll
-    for (int i = 0; i < DP; i += 4) {
-      const float4 v = *(const float4*)(sp + i);
-      S[i] = v.x; S[i + 1] = v.y; S[i + 2] = v.z; S[i + 3] = v.w;
+  for (int c = 0; c < COLS; ++c) {
+    if (MODE != 1 && j0 + c < dv) {
+#pragma unroll
+      for (int i = 0; i < DP; i += 4) {
+        const float4 v = *(const float4*)(sp + (size_t)c * parts * DP + i);
+        S[c][i] = v.x; S[c][i + 1] = v.y; S[c][i + 2] = v.z; S[c][i + 3] = v.w;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < DP; ++i) S[c][i] = 0.f;
     }
-  } else {
-#pragma unroll
-    for (int i = 0; i < DP; ++i) S[i] = 0.f;
   }
   const T* rows = (const T*)a.rows;
   const int wid = tid / WAVE, lane = tid % WAVE, nw = (blockDim.x + WAVE - 1) / WAVE;
   float loga_sum = 0.f;
-  const float zb = (tid < d && a.z_bias) ? a.z_bias[head * d + tid] : 0.f;
   for (int s0 = 0; s0 < n; s0 += STAGE) {
     const int ns = min(STAGE, n - s0);
-    // the stage's q, k and decays: thread i takes channel i of every token (all loads go out together)
-    if (tid < d) {
-      float zq[STAGE], kq[STAGE], qq[STAGE];
-#pragma unroll
-      for (int tt = 0; tt < STAGE; ++tt) {
-        const size_t t = (size_t)(t0 + s0 + min(tt, ns - 1));
-        zq[tt] = a.z[t * (size_t)(H * d) + head * d + tid];
-        kq[tt] = to_f(rows[t * a.ld + a.k_col + head * d + tid]);
-        qq[tt] = MODE == 1 ? 0.f : to_f(rows[t * a.ld + a.q_col + head * d + tid]);
-      }
-#pragma unroll
-      for (int tt = 0; tt < STAGE; ++tt) {
-        const float la_t = log_sigmoid(zq[tt] + zb) * a.inv_tau;
-        if (tt < ns) loga_sum += la_t;
-        la[tt * d + tid] = expf(la_t);
-        lk[tt * d + tid] = kq[tt];
-        lq[tt * d + tid] = qq[tt] * a.q_scale;
-      }
+    // the stage's q, k and decays: one (token, channel) a thread and trip, neighbouring threads on neighbouring channels
+    for (int it = tid; it < ns * d; it += blockDim.x) {
+      const int tt = it / d, ch = it - tt * d;
+      const size_t t = (size_t)(t0 + s0 + tt);
+      const float zq = a.z[t * (size_t)(H * d) + head * d + ch] + (a.z_bias ? a.z_bias[head * d + ch] : 0.f);
+      const float kq = to_f(rows[t * a.ld + a.k_col + head * d + ch]);
+      const float qq = MODE == 1 ? 0.f : to_f(rows[t * a.ld + a.q_col + head * d + ch]);
+      const float la_t = log_sigmoid(zq) * a.inv_tau;
+      if (MODE == 1) lg[it] = la_t;
+      la[it] = expf(la_t);
+      lk[it] = kq;
+      lq[it] = qq * a.q_scale;
     }
-    float vv[STAGE];
+    float vv[COLS][STAGE];
 #pragma unroll
-    for (int tt = 0; tt < STAGE; ++tt)
-      vv[tt] = (owner && tt < ns) ? to_f(rows[(size_t)(t0 + s0 + tt) * a.ld + a.v_col + head * dv + j]) : 0.f;
+    for (int c = 0; c < COLS; ++c)
+#pragma unroll
+      for (int tt = 0; tt < STAGE; ++tt)
+        vv[c][tt] = (j0 + c < dv && tt < ns) ? to_f(rows[(size_t)(t0 + s0 + tt) * a.ld + a.v_col + head * dv + j0 + c]) : 0.f;
     __syncthreads();
+    if (MODE == 1 && tid < d)
+      for (int tt = 0; tt < ns; ++tt) loga_sum += lg[tt * d + tid];
     for (int tt = 0; tt < ns; ++tt) {
       const float* aa = la + tt * d + p * DP;
       const float* kk = lk + tt * d + p * DP;
       const float* qv = lq + tt * d + p * DP;
-      const float v = vv[tt];
-      float acc = 0.f;
+      float acc[COLS];
+#pragma unroll
+      for (int c = 0; c < COLS; ++c) acc[c] = 0.f;
 #pragma unroll
       for (int i = 0; i < DP; ++i) {
         if (p * DP + i < d) {              // (uniform over the lanes that share p; DP divides into d for the usual sizes)
-          S[i] = fmaf(aa[i], S[i], kk[i] * v);
-          if (MODE != 1) acc = fmaf(S[i], qv[i], acc);
+          const float al = aa[i], kv = kk[i], qq = MODE != 1 ? qv[i] : 0.f;
+#pragma unroll
+          for (int c = 0; c < COLS; ++c) {
+            S[c][i] = fmaf(al, S[c][i], kv * vv[c][tt]);
+            if (MODE != 1) acc[c] = fmaf(S[c][i], qq, acc[c]);
+          }
         }
       }
       if (MODE != 1) {
-        for (int o = 1; o < parts; o <<= 1) acc += __shfl_xor(acc, o, WAVE);
-        if (owner && p == 0) lo[tt * dv + j] = acc;
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) {
+          float r = acc[c];
+          for (int o = 1; o < parts; o <<= 1) r += __shfl_xor(r, o, WAVE);
+          if (j0 + c < dv && p == 0) lo[tt * dv + j0 + c] = r;
+        }
       }
     }
     __syncthreads();
@@ -156,12 +167,17 @@ __global__ __launch_bounds__(GLA_MAX_THREADS(DP)) void gla_kernel(GlaArgs a) {
               from_f<T>(lo[tt * dv + c] * inv * load_dyn(a.norm_w, a.norm_dtype, c) * act_silu(g));
         }
       }
-      __syncthreads();
     }
+    __syncthreads();                       // (the next stage's loads overwrite what this stage read)
   }
-  if (MODE != 2 && owner) {
+  if (MODE != 2) {
 #pragma unroll
-    for (int i = 0; i < DP; i += 4) *(float4*)(sp + i) = make_float4(S[i], S[i + 1], S[i + 2], S[i + 3]);
+    for (int c = 0; c < COLS; ++c)
+      if (j0 + c < dv) {
+#pragma unroll
+        for (int i = 0; i < DP; i += 4)
+          *(float4*)(sp + (size_t)c * parts * DP + i) = make_float4(S[c][i], S[c][i + 1], S[c][i + 2], S[c][i + 3]);
+      }
   }
   if (MODE == 1 && tid < d) a.chunk_loga[(size_t)unit * H * d + head * d + tid] = loga_sum;
 }
@@ -198,19 +214,24 @@ __global__ __launch_bounds__(256) void gla_combine_kernel(CombineArgs a) {
 
 template <typename T, int DP>
 static int launch_gla(const GlaArgs& a, int R, int n_chunks, const int* req_chunk0, hipStream_t s) {
-  // (the first d threads load the stage's q, k and decays: a head of few values still gets a thread per key channel)
-  const int threads = ((max(a.dv * a.parts, a.d) + WAVE - 1) / WAVE) * WAVE;
+  // In one walk (steps of single tokens above all, which are bound by reading and writing S) a thread holds two columns of S
+  // where its registers allow (runs of up to 32 channels): 26 against 33 us for 64 requests of 16 heads x 64 x 128.  Chunks
+  // side by side are bound by the chain from token to token and want the waves: there two columns lost (167 against 144 us).
+  // The first d threads load the stage's q, k and decays, so a head of few values still gets a thread per key channel.
+  constexpr int COLS = DP <= 32 ? 2 : 1;
+  const auto threads_for = [&](int cols) { return ((max((a.dv + cols - 1) / cols * a.parts, a.d) + WAVE - 1) / WAVE) * WAVE; };
+  const int threads = threads_for(1);
   IFX_REQUIRE(threads <= GLA_MAX_THREADS(DP), "gla_scan: %d threads a head with %d channels each (at most %d)", threads, DP, GLA_MAX_THREADS(DP));
-  const size_t lds = (size_t)STAGE * (3 * a.d + a.dv) * sizeof(float);
+  const size_t lds = (size_t)STAGE * (4 * a.d + a.dv) * sizeof(float);
   if (n_chunks == 0) {
-    hipLaunchKernelGGL((gla_kernel<T, DP, 0>), dim3(R, a.H), dim3(threads), lds, s, a);
+    hipLaunchKernelGGL((gla_kernel<T, DP, 0, COLS>), dim3(R, a.H), dim3(threads_for(COLS)), lds, s, a);
     IFX_LAUNCH_CHECK();
   }
-  hipLaunchKernelGGL((gla_kernel<T, DP, 1>), dim3(n_chunks, a.H), dim3(threads), lds, s, a);
+  hipLaunchKernelGGL((gla_kernel<T, DP, 1, 1>), dim3(n_chunks, a.H), dim3(threads), lds, s, a);
   CombineArgs c{a.state, a.state_stride, a.state_offset, a.slots, req_chunk0, a.chunk_state, a.chunk_loga, a.H, a.d, a.dv, a.parts, DP};
   const size_t per = (size_t)a.H * a.dv * a.parts * DP;
   hipLaunchKernelGGL(gla_combine_kernel, dim3((unsigned)((per + 255) / 256), R), dim3(256), 0, s, c);
-  hipLaunchKernelGGL((gla_kernel<T, DP, 2>), dim3(n_chunks, a.H), dim3(threads), lds, s, a);
+  hipLaunchKernelGGL((gla_kernel<T, DP, 2, 1>), dim3(n_chunks, a.H), dim3(threads), lds, s, a);
   IFX_LAUNCH_CHECK();
 }
 
@@ -227,7 +248,7 @@ extern "C" int ifx_gla_scan(const void* rows, int dtype, int ld, int q_col, int 
   IFX_REQUIRE((state_offset % 4) == 0 && (state_stride % 4) == 0, "gla_scan: the state must lie at a multiple of 16 bytes");
   IFX_REQUIRE(state_stride >= state_offset + (long long)H * dv * parts * dp, "gla_scan: a state row of %lld floats is too short", state_stride);
   IFX_REQUIRE(n_chunks == 0 || (chunk_req && chunk_t0 && chunk_len && req_chunk0 && chunk_state && chunk_loga), "gla_scan: chunks without their lists");
-  IFX_REQUIRE((size_t)STAGE * (3 * d + dv) * sizeof(float) <= 64 * 1024, "gla_scan: d=%d, dv=%d need more LDS than a workgroup has", d, dv);
+  IFX_REQUIRE((size_t)STAGE * (4 * d + dv) * sizeof(float) <= 64 * 1024, "gla_scan: d=%d, dv=%d need more LDS than a workgroup has", d, dv);
   if (T == 0 || R == 0) return 0;
   GlaArgs a{rows, ld, q_col, k_col, v_col, g_col, z, z_bias, inv_tau, q_scale, eps, norm_w, norm_dtype, state,
             (size_t)state_stride, (size_t)state_offset, q_start, q_len, slots, out, H, d, dv, parts,

@@ -30,7 +30,7 @@ from .ffn import concat_weights
 from .plan import ParamSpec, StateSpec
 
 
-SCAN_CHUNK = 64             # rows of a chunk where long portions are cut into chunks that run side by side
+SCAN_CHUNK = 32             # rows of a chunk where long portions are cut into chunks that run side by side
 SCAN_CHUNK_MIN_ROWS = 128   # ... which happens in steps that bring some request this many rows or more
 
 
