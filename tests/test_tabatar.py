@@ -163,27 +163,27 @@ def test_window_attention_is_a_masked_softmax():
 
 
 def test_banded_frequencies_keep_short_waves_slow_long_ones_and_blend_between():
-    sc = {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 512}
-    f = pt.banded_frequencies(48, 250000.0, sc)
-    base = np.array([250000.0 ** (-2 * i / 48) for i in range(24)])
-    assert np.allclose(pt.banded_frequencies(48, 250000.0, None), base)
+    sc = {"factor": 6.0, "low": 1.0, "high": 3.0, "original": 1024}
+    f = pt.banded_frequencies(40, 30000.0, sc)
+    base = np.array([30000.0 ** (-2 * i / 40) for i in range(20)])
+    assert np.allclose(pt.banded_frequencies(40, 30000.0, None), base)
     wave = 2 * math.pi / base
-    kept, slowed = wave < 512 / 4.0, wave > 512 / 1.0
+    kept, slowed = wave < 1024 / 3.0, wave > 1024 / 1.0
     assert kept.any() and slowed.any() and (~kept & ~slowed).any()
-    assert np.allclose(f[kept], base[kept]) and np.allclose(f[slowed], base[slowed] / 8.0)
+    assert np.allclose(f[kept], base[kept]) and np.allclose(f[slowed], base[slowed] / 6.0)
     mid = ~kept & ~slowed
-    assert np.all(f[mid] < base[mid]) and np.all(f[mid] > base[mid] / 8.0) and list(f) == sorted(f, reverse=True)
+    assert np.all(f[mid] < base[mid]) and np.all(f[mid] > base[mid] / 6.0) and list(f) == sorted(f, reverse=True)
     # at the band's two ends the blend meets its neighbours
-    for wl, want in ((512 / 4.0, 1.0), (512 / 1.0, 1 / 8.0)):
-        s = (512 / wl - 1.0) / 3.0
-        assert np.isclose((1 - s) / 8.0 + s, want)
-    x = np.random.default_rng(1).normal(size=(3, 2, 54))
-    y = pt.rotate(x, np.array([0, 5, 900]), 48, 250000.0, sc)
-    assert np.allclose(y[0], x[0]) and np.allclose(y[..., 48:], x[..., 48:])
-    assert np.allclose(y[..., :24] ** 2 + y[..., 24:48] ** 2, x[..., :24] ** 2 + x[..., 24:48] ** 2)      # pair (i, i + dims/2) turns
+    for wl, want in ((1024 / 3.0, 1.0), (1024 / 1.0, 1 / 6.0)):
+        s = (1024 / wl - 1.0) / 2.0
+        assert np.isclose((1 - s) / 6.0 + s, want)
+    x = np.random.default_rng(1).normal(size=(3, 2, 46))
+    y = pt.rotate(x, np.array([0, 5, 900]), 40, 30000.0, sc)
+    assert np.allclose(y[0], x[0]) and np.allclose(y[..., 40:], x[..., 40:])
+    assert np.allclose(y[..., :20] ** 2 + y[..., 20:40] ** 2, x[..., :20] ** 2 + x[..., 20:40] ** 2)      # pair (i, i + dims/2) turns
     a = 5 * f[3]
-    assert np.allclose(y[1, 0, 3], x[1, 0, 3] * math.cos(a) - x[1, 0, 27] * math.sin(a))
-    assert np.allclose(y[1, 0, 27], x[1, 0, 27] * math.cos(a) + x[1, 0, 3] * math.sin(a))
+    assert np.allclose(y[1, 0, 3], x[1, 0, 3] * math.cos(a) - x[1, 0, 23] * math.sin(a))
+    assert np.allclose(y[1, 0, 23], x[1, 0, 23] * math.cos(a) + x[1, 0, 3] * math.sin(a))
 
 
 def test_the_recurrence_is_attention_with_decayed_keys_and_carries_on_from_its_state():
