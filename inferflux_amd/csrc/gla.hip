@@ -212,30 +212,48 @@ __global__ __launch_bounds__(256) void gla_combine_kernel(CombineArgs a) {
   *slot = S;
 }
 
+template <typename T, int DP, int MODE, int COLS>
+static void launch_gla_mode(const GlaArgs& a, int units, int threads, size_t lds, hipStream_t s) {
+  hipLaunchKernelGGL((gla_kernel<T, DP, MODE, COLS>), dim3(units, a.H), dim3(threads), lds, s, a);
+}
+
+// A launch of MODE with ``cols`` columns of S a thread (1, 2 or 4; what DP allows is checked by the caller).
+template <typename T, int DP, int MODE>
+static void launch_gla_cols(const GlaArgs& a, int units, int cols, int threads, size_t lds, hipStream_t s) {
+  if constexpr (DP <= 16) { if (cols == 4) return launch_gla_mode<T, DP, MODE, 4>(a, units, threads, lds, s); }
+  if constexpr (DP <= 32) { if (cols == 2) return launch_gla_mode<T, DP, MODE, 2>(a, units, threads, lds, s); }
+  launch_gla_mode<T, DP, MODE, 1>(a, units, threads, lds, s);
+}
+
 template <typename T, int DP>
 static int launch_gla(const GlaArgs& a, int R, int n_chunks, const int* req_chunk0, hipStream_t s) {
-  // In one walk (steps of single tokens above all, which are bound by reading and writing S) a thread holds two columns of S
-  // where its registers allow (runs of up to 32 channels): 26 against 33 us for 64 requests of 16 heads x 64 x 128.  Chunks
-  // side by side are bound by the chain from token to token and want the waves: there two columns lost (167 against 144 us).
-  // The first d threads load the stage's q, k and decays, so a head of few values still gets a thread per key channel.
-  constexpr int COLS = DP <= 32 ? 2 : 1;
+  // A thread holds 1, 2 or 4 columns of S as its registers allow (4 for runs of 16 channels, 2 for 32).  In one walk (steps
+  // of single tokens above all, which are bound by reading and writing S) two where possible: 26 against 33 us for 64 requests
+  // of 16 heads x 64 x 128.  Chunks side by side are bound by the chain from token to token and want the waves: there two
+  // columns lost (167 against 144 us), so they take as few as fit a workgroup.  The first d threads also load, so a head of
+  // few values still gets a thread per key channel.
+  constexpr int MAX_COLS = DP <= 16 ? 4 : (DP <= 32 ? 2 : 1);
   const auto threads_for = [&](int cols) { return ((max((a.dv + cols - 1) / cols * a.parts, a.d) + WAVE - 1) / WAVE) * WAVE; };
-  const int threads = threads_for(1);
-  IFX_REQUIRE(threads <= GLA_MAX_THREADS(DP), "gla_scan: %d threads a head with %d channels each (at most %d)", threads, DP, GLA_MAX_THREADS(DP));
+  int cols_chunk = 1;
+  while (cols_chunk < MAX_COLS && threads_for(cols_chunk) > GLA_MAX_THREADS(DP)) cols_chunk *= 2;
+  const int cols_walk = max(cols_chunk, min(2, MAX_COLS));
+  IFX_REQUIRE(threads_for(cols_chunk) <= GLA_MAX_THREADS(DP), "gla_scan: %d threads a head with %d channels each (at most %d)",
+              threads_for(cols_chunk), DP, GLA_MAX_THREADS(DP));
   const size_t lds = (size_t)STAGE * (4 * a.d + a.dv) * sizeof(float);
   if (n_chunks == 0) {
-    hipLaunchKernelGGL((gla_kernel<T, DP, 0, COLS>), dim3(R, a.H), dim3(threads_for(COLS)), lds, s, a);
+    launch_gla_cols<T, DP, 0>(a, R, cols_walk, threads_for(cols_walk), lds, s);
     IFX_LAUNCH_CHECK();
   }
-  hipLaunchKernelGGL((gla_kernel<T, DP, 1, 1>), dim3(n_chunks, a.H), dim3(threads), lds, s, a);
+  launch_gla_cols<T, DP, 1>(a, n_chunks, cols_chunk, threads_for(cols_chunk), lds, s);
   CombineArgs c{a.state, a.state_stride, a.state_offset, a.slots, req_chunk0, a.chunk_state, a.chunk_loga, a.H, a.d, a.dv, a.parts, DP};
   const size_t per = (size_t)a.H * a.dv * a.parts * DP;
   hipLaunchKernelGGL(gla_combine_kernel, dim3((unsigned)((per + 255) / 256), R), dim3(256), 0, s, c);
-  hipLaunchKernelGGL((gla_kernel<T, DP, 2, 1>), dim3(n_chunks, a.H), dim3(threads), lds, s, a);
+  launch_gla_cols<T, DP, 2>(a, n_chunks, cols_chunk, threads_for(cols_chunk), lds, s);
   IFX_LAUNCH_CHECK();
 }
 
-// dp: channels a thread holds (16, 32, 64 or 128); parts: a power of two with parts * dp >= d and dv * parts <= 1024.
+// dp: channels a thread holds (16, 32, 64 or 128); parts: a power of two with parts * dp >= d; a head's columns, 1-4 a thread,
+// times parts must fit a workgroup.
 extern "C" int ifx_gla_scan(const void* rows, int dtype, int ld, int q_col, int k_col, int v_col, int g_col, const float* z,
                             const float* z_bias, float inv_tau, float q_scale, float eps, const void* norm_w, int norm_dtype,
                             float* state, long long state_stride, long long state_offset, const int* q_start, const int* q_len,
@@ -244,7 +262,7 @@ extern "C" int ifx_gla_scan(const void* rows, int dtype, int ld, int q_col, int 
                             const int* req_chunk0, float* chunk_state, float* chunk_loga, void* stream) {
   IFX_REQUIRE(T >= 0 && R >= 0 && H > 0 && d > 0 && dv > 0, "gla_scan: bad sizes T=%d R=%d H=%d d=%d dv=%d", T, R, H, d, dv);
   IFX_REQUIRE(parts > 0 && (parts & (parts - 1)) == 0 && parts <= WAVE && parts * dp >= d, "gla_scan: %d parts of %d channels for d=%d", parts, dp, d);
-  IFX_REQUIRE(dv * parts <= 1024 && d <= 1024, "gla_scan: a head of %d values x %d parts does not fit a workgroup", dv, parts);
+  IFX_REQUIRE(d <= 1024, "gla_scan: a head of %d key channels does not fit a workgroup", d);
   IFX_REQUIRE((state_offset % 4) == 0 && (state_stride % 4) == 0, "gla_scan: the state must lie at a multiple of 16 bytes");
   IFX_REQUIRE(state_stride >= state_offset + (long long)H * dv * parts * dp, "gla_scan: a state row of %lld floats is too short", state_stride);
   IFX_REQUIRE(n_chunks == 0 || (chunk_req && chunk_t0 && chunk_len && req_chunk0 && chunk_state && chunk_loga), "gla_scan: chunks without their lists");

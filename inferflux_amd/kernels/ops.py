@@ -1179,12 +1179,21 @@ GLA_THREAD_CHANNELS = ((16, 512), (32, 1024), (64, 512), (128, 256))   # channel
 
 def gla_layout(d: int, dv: int) -> Tuple[int, int]:
     """(channels a thread holds, threads per column) for a head of d key channels and dv values: the first pairing whose
-    workgroup (dv columns times the threads of a column) fits.  A request's S takes heads * dv * parts * channels floats."""
-    for dp, max_threads in GLA_THREAD_CHANNELS:
+    workgroup (dv columns times the threads of a column) fits; failing that, the first in which a thread holds several
+    columns (4 with 16 channels, 2 with 32: what its registers take).  A request's S takes heads * dv * parts * channels
+    floats."""
+    def parts_for(dp):
         parts = 1
         while parts * dp < d:
             parts *= 2
+        return parts
+    for dp, max_threads in GLA_THREAD_CHANNELS:
+        parts = parts_for(dp)
         if parts <= 64 and max(dv * parts, d) <= max_threads:     # (a thread per key channel loads a stage's q, k and decays)
+            return dp, parts
+    for dp, cols in ((16, 4), (32, 2)):
+        parts = parts_for(dp)
+        if parts <= 64 and max(-(-dv // cols) * parts, d) <= 1024:
             return dp, parts
     raise KernelError(f"gla: a head of {d} key channels and {dv} values does not fit a workgroup")
 

@@ -220,7 +220,8 @@ def test_elementwise_sigmoid_gate_from_the_projected_rows(dtype, T, C, ld, col):
 
 
 GLA_SHAPES = [(2, 16, 24, 8.0), (3, 8, 16, 3.0), (1, 32, 8, 20.0), (2, 12, 12, 1.0), (4, 64, 64, 16.0), (3, 10, 14, 5.0), (4, 128, 128, 16.0),
-              (8, 32, 96, 4.0), (2, 48, 256, 2.0), (1, 200, 16, 9.0), (2, 128, 256, 16.0), (3, 128, 8, 1.0), (1, 300, 4, 2.0)]
+              (8, 32, 96, 4.0), (2, 48, 256, 2.0), (1, 200, 16, 9.0), (2, 128, 256, 16.0), (3, 128, 8, 1.0), (1, 300, 4, 2.0),
+              (2, 192, 192, 4.0), (1, 256, 256, 8.0), (1, 96, 512, 2.0)]       # (the last three: several columns of S a thread)
 
 
 def _gla_inputs(seed, T, H, d, dv, dt, extra=5):
@@ -282,7 +283,7 @@ def test_gated_linear_attention_over_steps_with_state_in_slots(dtype, H, d, dv, 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("H,d,dv,tau,chunk", [(2, 16, 24, 8.0, 64), (3, 8, 16, 3.0, 16), (4, 64, 64, 16.0, 64), (3, 10, 14, 5.0, 7), (2, 128, 128, 16.0, 64),
-                                             (1, 32, 8, 20.0, 200)])
+                                             (1, 32, 8, 20.0, 200), (1, 192, 192, 8.0, 32), (1, 256, 256, 4.0, 64)])
 def test_gated_linear_attention_in_chunks_side_by_side(dtype, H, d, dv, tau, chunk):
     """Long portions cut into chunks that first run from zero and then from what the chunks before them leave: the same
     outputs and the same final state as the walk in one piece, for requests of unequal length that start from a state."""
