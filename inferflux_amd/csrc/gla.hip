@@ -227,16 +227,16 @@ static void launch_gla_cols(const GlaArgs& a, int units, int cols, int threads, 
 
 template <typename T, int DP>
 static int launch_gla(const GlaArgs& a, int R, int n_chunks, const int* req_chunk0, hipStream_t s) {
-  // A thread holds 1, 2 or 4 columns of S as its registers allow (4 for runs of 16 channels, 2 for 32).  In one walk (steps
-  // of single tokens above all, which are bound by reading and writing S) two where possible: 26 against 33 us for 64 requests
-  // of 16 heads x 64 x 128.  Chunks side by side are bound by the chain from token to token and want the waves: there two
-  // columns lost (167 against 144 us), so they take as few as fit a workgroup.  The first d threads also load, so a head of
-  // few values still gets a thread per key channel.
+  // A thread holds 1, 2 or 4 columns of S as its registers allow (4 for runs of 16 channels, 2 for 32): what it reads of a
+  // token's q, k and decays from LDS then serves several columns.  Two where possible (steps of single tokens, which are bound
+  // by reading and writing S: 23 against 33 us for 64 requests of 16 heads x 64 x 128; chunks side by side: 86 + 64 against
+  // 95 + 67 us for 2,048 rows), more only where a head's columns would not fit a workgroup otherwise.  The first d threads also
+  // load, so a head of few values still gets a thread per key channel.
   constexpr int MAX_COLS = DP <= 16 ? 4 : (DP <= 32 ? 2 : 1);
   const auto threads_for = [&](int cols) { return ((max((a.dv + cols - 1) / cols * a.parts, a.d) + WAVE - 1) / WAVE) * WAVE; };
-  int cols_chunk = 1;
+  int cols_chunk = min(2, MAX_COLS);
   while (cols_chunk < MAX_COLS && threads_for(cols_chunk) > GLA_MAX_THREADS(DP)) cols_chunk *= 2;
-  const int cols_walk = max(cols_chunk, min(2, MAX_COLS));
+  const int cols_walk = cols_chunk;
   IFX_REQUIRE(threads_for(cols_chunk) <= GLA_MAX_THREADS(DP), "gla_scan: %d threads a head with %d channels each (at most %d)",
               threads_for(cols_chunk), DP, GLA_MAX_THREADS(DP));
   const size_t lds = (size_t)STAGE * (4 * a.d + a.dv) * sizeof(float);
