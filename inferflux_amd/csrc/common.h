@@ -94,14 +94,22 @@ __device__ __forceinline__ float block_max(float v, float* red) {
 
 // Gated activations of a feed-forward, act(gate) * up, in float.  ACT_SILU: gate / (1 + exp(-gate)); ACT_GELU_TANH:
 // 0.5 gate (1 + tanh(sqrt(2 / pi) (gate + 0.044715 gate^3))).  As a product's epilogue they are EPI 1 and EPI 3.
+// ACT_CLAMPED_SWISH (with a limit L): g = min(gate, L), u = clamp(up, -L, L); g sigmoid(1.702 g) (u + 1).
 #define ACT_SILU 0
 #define ACT_GELU_TANH 1
+#define ACT_CLAMPED_SWISH 2
 __device__ __forceinline__ float act_silu(float g) { return g / (1.0f + expf(-g)); }
 __device__ __forceinline__ float act_gelu_tanh(float g) {
   return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
 }
 __device__ __forceinline__ float gated_act(float g, float up, int act) {
   return (act == ACT_GELU_TANH ? act_gelu_tanh(g) : act_silu(g)) * up;
+}
+__device__ __forceinline__ float gated_act(float g, float up, int act, float limit) {
+  if (act != ACT_CLAMPED_SWISH) return gated_act(g, up, act);
+  g = fminf(g, limit);
+  up = fminf(fmaxf(up, -limit), limit);
+  return g / (1.0f + expf(-1.702f * g)) * (up + 1.0f);
 }
 template <int EPI> __device__ __forceinline__ float gated_epilogue(float g, float up) {
   return (EPI == 3 ? act_gelu_tanh(g) : act_silu(g)) * up;

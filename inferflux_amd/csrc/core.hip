@@ -777,21 +777,22 @@ extern "C" int ifx_rope_append(const void* qkv, int dtype, const void* bias, int
 }
 
 // ---------------------------------------------------------------------------------------
-// out[t, i] = act(gate) * up (act: ACT_SILU gate / (1 + exp(-gate)), ACT_GELU_TANH the tanh form of gelu), with gu[t] = [gate (I) | up (I)] or, interleaved,
+// out[t, i] = act(gate) * up (act: ACT_SILU gate / (1 + exp(-gate)), ACT_GELU_TANH the tanh form of gelu; ACT_CLAMPED_SWISH
+// with its limit: common.h), with gu[t] = [gate (I) | up (I)] or, interleaved,
 // gu[t] = [gate_0, up_0, gate_1, up_1, ...].
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t n, int interleaved, int act) {
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t n, int interleaved, int act, float limit) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= n) return;
   const size_t t = idx / I;
   const int i = (int)(idx % I);
   const float g = to_f(gu[t * 2 * I + (interleaved ? 2 * i : i)]);
   const float u = to_f(gu[t * 2 * I + (interleaved ? 2 * i + 1 : I + i)]);
-  out[idx] = from_f<T>(gated_act(g, u, act));
+  out[idx] = from_f<T>(gated_act(g, u, act, limit));
 }
 
 // The interleaved bf16 case in 32-byte pieces: 8 gate/up pairs in, 8 results out (I a multiple of 8).
-__global__ void swiglu_pairs_bf16_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, size_t n8, int act) {
+__global__ void swiglu_pairs_bf16_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, size_t n8, int act, float limit) {
   typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n8) return;
@@ -800,27 +801,27 @@ __global__ void swiglu_pairs_bf16_kernel(const bf16_t* __restrict__ gu, bf16_t* 
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     const float g0 = (float)a[2 * e], u0 = (float)a[2 * e + 1], g1 = (float)b[2 * e], u1 = (float)b[2 * e + 1];
-    o[e] = (__bf16)gated_act(g0, u0, act);
-    o[e + 4] = (__bf16)gated_act(g1, u1, act);
+    o[e] = (__bf16)gated_act(g0, u0, act, limit);
+    o[e + 4] = (__bf16)gated_act(g1, u1, act, limit);
   }
   *(bf16x8*)(out + 8 * i) = o;
 }
 
-extern "C" int ifx_swiglu(const void* gu, void* out, int dtype, int T, int I, int interleaved, int act, void* stream) {
-  IFX_REQUIRE(act == ACT_SILU || act == ACT_GELU_TANH, "gated activation: unknown kind %d", act);
+extern "C" int ifx_swiglu(const void* gu, void* out, int dtype, int T, int I, int interleaved, int act, float limit, void* stream) {
+  IFX_REQUIRE(act == ACT_SILU || act == ACT_GELU_TANH || (act == ACT_CLAMPED_SWISH && limit > 0.f), "gated activation: unknown kind %d (limit %g)", act, (double)limit);
   IFX_REQUIRE(T >= 0 && I > 0, "swiglu: bad sizes T=%d I=%d", T, I);
   if (T == 0) return 0;
   const size_t n = (size_t)T * I;
   if (interleaved && dtype == DT_BF16 && I % 8 == 0) {
     const size_t n8 = n / 8;
     hipLaunchKernelGGL(swiglu_pairs_bf16_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                       (const bf16_t*)gu, (bf16_t*)out, n8, act);
+                       (const bf16_t*)gu, (bf16_t*)out, n8, act, limit);
     IFX_LAUNCH_CHECK();
   }
   const unsigned blocks = (unsigned)((n + 255) / 256);
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == DT_F32) hipLaunchKernelGGL(swiglu_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)gu, (float*)out, I, n, interleaved, act);
-  else if (dtype == DT_BF16) hipLaunchKernelGGL(swiglu_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, (const bf16_t*)gu, (bf16_t*)out, I, n, interleaved, act);
+  if (dtype == DT_F32) hipLaunchKernelGGL(swiglu_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)gu, (float*)out, I, n, interleaved, act, limit);
+  else if (dtype == DT_BF16) hipLaunchKernelGGL(swiglu_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, (const bf16_t*)gu, (bf16_t*)out, I, n, interleaved, act, limit);
   else IFX_FAIL("swiglu: unknown dtype %d", dtype);
   IFX_LAUNCH_CHECK();
 }

@@ -10,6 +10,9 @@
 //   ifx_moe_down_grouped      parts[choice][row] = weight[item] * Wd[e] act[item] in float: the choices of a row are
 //                      the "slices" of a sum that the kernel which adds the result to the stream takes in order, so a
 //                      row's result does not depend on where its items lay in the order
+//                      An expert from `n_real` upwards is an identity expert without weights: the first product leaves its
+//                      tiles alone and the second writes weight[item] * x[row] (`identity`, the rows as the first product
+//                      read them; N is then the rows' width).  The first product's activation is `act` of common.h.
 //   ifx_headwise_grouped      out[t][h][:N] = W[h] x[t][h], tiles of TM rows of one head
 //
 // One kernel does all three products.  A workgroup of four waves takes TM = 64 or 128 items and TN = 128 weight rows;
@@ -91,6 +94,9 @@ struct GroupedArgs {
   int K, NW, x_div, x_row, x_group;
   int T, top;               // MODE_DOWN: parts [top][T][NW]; MODE_HEADS: T rows, tiles_per_group = ceil(T / TM)
   int out_head, n_groups;   // MODE_HEADS: out [T][n_groups][out_head]
+  int n_real;               // experts with weights; tiles of later ones are identity experts' (not MODE_HEADS)
+  const bf16_t* identity;   // MODE_DOWN: [T][NW], what an identity expert hands back
+  int act; float limit;     // MODE_GATE_UP: the activation
 };
 
 // MT: tiles of 32 items per wave (1: the workgroup takes 64 items, 2: 128)
@@ -115,6 +121,15 @@ __global__ __launch_bounds__(256) void grouped_kernel(GroupedArgs a) {
     count = min(a.tile_count[tile], BM);
   }
   const int n0 = blockIdx.y * TN;
+  if (MODE != MODE_HEADS && group >= a.n_real) {        // an identity expert's tile (the whole workgroup)
+    if (MODE == MODE_DOWN)
+      for (int x = tid; x < count * TN; x += 256) {
+        const int m = a.sorted[start + x / TN], n = n0 + x % TN;
+        if (n < a.NW)
+          ((float*)a.out)[((size_t)(m % a.top) * a.T + m / a.top) * a.NW + n] = a.weights[m] * (float)a.identity[(size_t)(m / a.top) * a.NW + n];
+      }
+    return;
+  }
   for (int i = tid; i < BM; i += 256) items[i] = i < count ? (MODE == MODE_HEADS ? start + i : a.sorted[start + i]) : -1;
   __syncthreads();
   const int wave = tid / WAVE, lane = tid % WAVE, l32 = lane & 31, hi = lane >> 5;
@@ -197,7 +212,7 @@ __global__ __launch_bounds__(256) void grouped_kernel(GroupedArgs a) {
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const float g = acc[mt][nt][4 * q + r], u = acc[mt][nt][8 + 4 * q + r];
-            y[r] = (__bf16)(g / (1.0f + expf(-g)) * u);
+            y[r] = (__bf16)gated_act(g, u, a.act, a.limit);
           }
           *(bf16x4*)(act + f) = y;
         }
@@ -242,11 +257,11 @@ static int check_common(int K, int x_row, int x_group) {
 // act [n_items][ff] (bfloat16) from x [T][K] and the paired weights w [E][2 ff][K]; item i is row i / top.
 extern "C" int ifx_moe_gate_up_grouped(const void* x, const void* w, void* act, const int* sorted, const int* tile_expert,
                                        const int* tile_start, const int* tile_count, const int* n_tiles, int max_tiles, int tile_items,
-                                       int K, int ff, int top, void* stream) {
+                                       int K, int ff, int top, int n_real, int act_kind, float limit, void* stream) {
   IFX_REQUIRE(check_common(K, K, 0) && ff > 0 && ff % 16 == 0 && top > 0, "moe_gate_up_grouped: K=%d must be a multiple of 8, ff=%d of 16", K, ff);
   if (max_tiles <= 0) return 0;
   GroupedArgs a{(const bf16_t*)x, (const bf16_t*)w, act, sorted, tile_expert, tile_start, tile_count, n_tiles, nullptr,
-                K, 2 * ff, top, K, 0, 0, top, 0, 0};
+                K, 2 * ff, top, K, 0, 0, top, 0, 0, n_real, nullptr, act_kind, limit};
   const dim3 grid(max_tiles, (2 * ff + TN - 1) / TN);
   if (tile_items == 128) hipLaunchKernelGGL((grouped_kernel<MODE_GATE_UP, 2>), grid, dim3(256), 0, (hipStream_t)stream, a);
   else if (tile_items == 64) hipLaunchKernelGGL((grouped_kernel<MODE_GATE_UP, 1>), grid, dim3(256), 0, (hipStream_t)stream, a);
@@ -257,11 +272,12 @@ extern "C" int ifx_moe_gate_up_grouped(const void* x, const void* w, void* act, 
 // parts [top][T][N] (float) = weights[item] * (Wd[e] act[item]), w [E][N][ff]
 extern "C" int ifx_moe_down_grouped(const void* act, const void* w, float* parts, const float* weights, const int* sorted,
                                     const int* tile_expert, const int* tile_start, const int* tile_count, const int* n_tiles,
-                                    int max_tiles, int tile_items, int T, int N, int ff, int top, void* stream) {
+                                    int max_tiles, int tile_items, int T, int N, int ff, int top, int n_real, const void* identity,
+                                    void* stream) {
   IFX_REQUIRE(check_common(ff, ff, 0) && N > 0 && top > 0 && T >= 0, "moe_down_grouped: ff=%d must be a multiple of 8", ff);
   if (max_tiles <= 0 || T == 0) return 0;
   GroupedArgs a{(const bf16_t*)act, (const bf16_t*)w, parts, sorted, tile_expert, tile_start, tile_count, n_tiles, weights,
-                ff, N, 1, ff, 0, T, top, 0, 0};
+                ff, N, 1, ff, 0, T, top, 0, 0, n_real, (const bf16_t*)identity, 0, 0.f};
   const dim3 grid(max_tiles, (N + TN - 1) / TN);
   if (tile_items == 128) hipLaunchKernelGGL((grouped_kernel<MODE_DOWN, 2>), grid, dim3(256), 0, (hipStream_t)stream, a);
   else if (tile_items == 64) hipLaunchKernelGGL((grouped_kernel<MODE_DOWN, 1>), grid, dim3(256), 0, (hipStream_t)stream, a);
@@ -275,7 +291,7 @@ extern "C" int ifx_headwise_grouped(const void* x, const void* w, void* out, int
   IFX_REQUIRE(check_common(K, x_row, x_head) && N > 0 && H > 0 && out_head >= N, "headwise_grouped: K=%d, the rows of x (%d) and its heads (%d) must be multiples of 8", K, x_row, x_head);
   if (T <= 0) return 0;
   GroupedArgs a{(const bf16_t*)x, (const bf16_t*)w, out, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
-                K, N, 1, x_row, x_head, T, 1, out_head, H};
+                K, N, 1, x_row, x_head, T, 1, out_head, H, H, nullptr, 0, 0.f};
   if (T > 64) hipLaunchKernelGGL((grouped_kernel<MODE_HEADS, 2>), dim3(((T + 127) / 128) * H, (N + TN - 1) / TN), dim3(256), 0, (hipStream_t)stream, a);
   else hipLaunchKernelGGL((grouped_kernel<MODE_HEADS, 1>), dim3(((T + 63) / 64) * H, (N + TN - 1) / TN), dim3(256), 0, (hipStream_t)stream, a);
   IFX_LAUNCH_CHECK();

@@ -4,10 +4,13 @@
 //                     to the product kernels), score s = sigmoid(z) (or softmax over the experts), choice of `top` experts
 //                     among those of the best `keep` of `groups` equal groups of neighbouring experts (a group's
 //                     score: the sum of its `group_top` largest scores); the weights are the chosen scores as they
-//                     are or divided by their sum.  Writes ids [T][top] (int32) and weights [T][top] (float), in
+//                     are or divided by their sum.  With `choice_bias` [E] the choice (of groups and of experts) goes by
+//                     s + choice_bias while the weights stay the scores s themselves.  Writes ids [T][top] (int32) and weights [T][top] (float), in
 //                     descending order of score, the lower index first among equals.
-//   ifx_moe_gate_up   a[t][j][:] = silu(Wg[e] h_t) * (Wu[e] h_t) for e = ids[t][j]       (Wg, Wu [E][ff][K])
+//   ifx_moe_gate_up   a[t][j][:] = act(Wg[e] h_t, Wu[e] h_t) for e = ids[t][j]          (Wg, Wu [E][ff][K]; act: common.h)
 //   ifx_moe_down      out[t][:] = sum_j weights[t][j] * Wd[e_j] a[t][j][:]              (Wd [E][N][ff])
+//                     An id from `n_real` upwards names an identity expert, which has no weights: its output is the
+//                     row h_t itself (ifx_moe_gate_up leaves such items alone, ifx_moe_down adds weights[t][j] * h_t).
 //
 // The two product kernels read the expert of every (row, choice) from device memory, so their grid depends on the
 // step's layout alone.  One wave forms one output element at a time (lanes across k, the fixed-order sum of
@@ -68,11 +71,13 @@ struct RouteArgs {
   int T, K, E, top, groups, keep, group_top, softmax, renorm;
   float scale;
   const float* bias;     // [E] added to the logits, or null
+  const float* choice_bias;   // [E] added to the scores for the choice alone, or null
 };
 
 template <typename T>
 __global__ __launch_bounds__(1024) void moe_route_kernel(RouteArgs a) {
   __shared__ float s[MAX_EXPERTS];       // scores
+  __shared__ float c[MAX_EXPERTS];       // what the choice goes by: the scores, plus the choice's bias
   __shared__ float gs[MAX_EXPERTS + MAX_TOP];      // group scores, and behind them the chosen scores in order
   __shared__ int shut[MAX_EXPERTS];      // 1: a group that is shut out
   __shared__ float red[16];
@@ -120,6 +125,8 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(RouteArgs a) {
     for (int e = threadIdx.x; e < a.E; e += blockDim.x) s[e] = 1.0f / (1.0f + expf(-s[e]));
   }
   __syncthreads();
+  for (int e = threadIdx.x; e < a.E; e += blockDim.x) c[e] = a.choice_bias ? s[e] + a.choice_bias[e] : s[e];
+  __syncthreads();
   // Every thread ranks what it owns among its like (more of them score higher, or as high at a lower index): a group
   // among the groups, then an expert among the experts of the groups that are kept.  The rank is the place in the output.
   const int per = a.E / a.groups;
@@ -132,10 +139,10 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(RouteArgs a) {
         for (int e = g * per; e < (g + 1) * per; ++e) {
           bool used = false;
           for (int q = 0; q < r; ++q) used |= taken[q] == e;
-          if (!used && (best < 0 || s[e] > s[best])) best = e;
+          if (!used && (best < 0 || c[e] > c[best])) best = e;
         }
         taken[r] = best;
-        sum += s[best];
+        sum += c[best];
       }
     }
     gs[g] = sum;
@@ -151,7 +158,7 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(RouteArgs a) {
   for (int e = threadIdx.x; e < a.E; e += blockDim.x) {
     if (shut[e / per]) continue;
     int rank = 0;
-    for (int o = 0; o < a.E; ++o) rank += (!shut[o / per] && (s[o] > s[e] || (s[o] == s[e] && o < e))) ? 1 : 0;
+    for (int o = 0; o < a.E; ++o) rank += (!shut[o / per] && (c[o] > c[e] || (c[o] == c[e] && o < e))) ? 1 : 0;
     if (rank < a.top) {
       a.ids[t * a.top + rank] = e;
       gs[a.groups + rank] = s[e];        // (gs has room behind the groups: E >= groups + top is not needed, MAX_EXPERTS + ... see below)
@@ -167,14 +174,14 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(RouteArgs a) {
 }
 
 extern "C" int ifx_moe_route(const void* h, const void* w, int dtype, const float* z, int* ids, float* weights, int T, int K, int E,
-                             int top, int groups, int keep, int group_top, int softmax, int renorm, float scale, const float* bias, void* stream) {
+                             int top, int groups, int keep, int group_top, int softmax, int renorm, float scale, const float* bias, const float* choice_bias, void* stream) {
   IFX_REQUIRE(z || (h && w), "moe_route: neither logits nor the rows and the router's weight");
   IFX_REQUIRE(T >= 0 && K > 0 && E > 0 && E <= MAX_EXPERTS, "moe_route: %d experts (at most %d), K=%d", E, MAX_EXPERTS, K);
   IFX_REQUIRE(groups > 0 && E % groups == 0 && keep > 0 && keep <= groups, "moe_route: %d experts in %d groups of which %d are kept", E, groups, keep);
   IFX_REQUIRE(group_top > 0 && group_top <= 8, "moe_route: a group's score sums its %d largest (1-8)", group_top);
   IFX_REQUIRE(top > 0 && top <= MAX_TOP && top <= keep * (E / groups), "moe_route: top %d of %d x %d experts", top, keep, E / groups);
   if (T == 0) return 0;
-  RouteArgs a{h, w, z, ids, weights, T, K, E, top, groups, keep, group_top, softmax, renorm, scale, bias};
+  RouteArgs a{h, w, z, ids, weights, T, K, E, top, groups, keep, group_top, softmax, renorm, scale, bias, choice_bias};
   // a wave takes four experts at a time: as many waves as that takes, up to 16 (the scores are a chain of trips to memory otherwise)
   const int threads = z ? WAVE * (E <= 64 ? 1 : 4) : WAVE * (E <= 16 ? 4 : (E <= 32 ? 8 : 16));
   hipStream_t s = (hipStream_t)stream;
@@ -191,10 +198,12 @@ extern "C" int ifx_moe_route(const void* h, const void* w, int dtype, const floa
 template <typename T>
 __global__ __launch_bounds__(WAVE * WAVES) void moe_gate_up_kernel(const T* __restrict__ h, const T* __restrict__ wg,
                                                                    const T* __restrict__ wu, const int* __restrict__ ids,
-                                                                   T* __restrict__ act, int K, int ff, int top, int paired) {
+                                                                   T* __restrict__ act, int K, int ff, int top, int paired,
+                                                                   int n_real, int act_kind, float limit) {
   const size_t item = blockIdx.x;                 // (row, choice)
   const size_t t = item / top;
   const int e = ids[item];
+  if (e >= n_real) return;                        // an identity expert: nothing to form (the whole workgroup leaves)
   const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const T* x = h + t * K;
   const int i0 = (blockIdx.y * WAVES + wid) * ROWS_PER_WAVE;
@@ -229,14 +238,15 @@ __global__ __launch_bounds__(WAVE * WAVES) void moe_gate_up_kernel(const T* __re
 #pragma unroll
   for (int r = 0; r < ROWS_PER_WAVE; ++r) {
     const float sg = wave_sum(sum[2 * r]), su = wave_sum(sum[2 * r + 1]);
-    if (lane == 0 && i0 + r < ff) act[item * ff + i0 + r] = from_f<T>(sg / (1.0f + expf(-sg)) * su);
+    if (lane == 0 && i0 + r < ff) act[item * ff + i0 + r] = from_f<T>(gated_act(sg, su, act_kind, limit));
   }
 }
 
 template <typename T>
 __global__ __launch_bounds__(WAVE * WAVES) void moe_down_kernel(const T* __restrict__ act, const T* __restrict__ wd,
                                                                 const int* __restrict__ ids, const float* __restrict__ weights,
-                                                                T* __restrict__ out, int N, int ff, int top) {
+                                                                T* __restrict__ out, int N, int ff, int top, int n_real,
+                                                                const T* __restrict__ h) {
   const size_t t = blockIdx.x;
   const int wid = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int n0 = (blockIdx.y * WAVES + wid) * ROWS_PER_WAVE;
@@ -246,6 +256,11 @@ __global__ __launch_bounds__(WAVE * WAVES) void moe_down_kernel(const T* __restr
   for (int r = 0; r < ROWS_PER_WAVE; ++r) y[r] = 0.f;
   for (int j = 0; j < top; ++j) {
     const int e = ids[t * top + j];
+    if (e >= n_real) {          // an identity expert: the row itself (N is the row's width)
+#pragma unroll
+      for (int r = 0; r < ROWS_PER_WAVE; ++r) y[r] = fmaf(weights[t * top + j], to_f(h[t * N + min(n0 + r, N - 1)]), y[r]);
+      continue;
+    }
     const T* a = act + (t * top + j) * ff;
     float sum[ROWS_PER_WAVE];
     if (ff % 8 == 0) {
@@ -272,30 +287,31 @@ __global__ __launch_bounds__(WAVE * WAVES) void moe_down_kernel(const T* __restr
 }
 
 extern "C" int ifx_moe_gate_up(const void* h, const void* wg, const void* wu, const int* ids, void* act, int dtype, int T, int K,
-                               int ff, int top, int paired, void* stream) {
+                               int ff, int top, int paired, int n_real, int act_kind, float limit, void* stream) {
   IFX_REQUIRE(T >= 0 && K > 0 && ff > 0 && top > 0, "moe_gate_up: bad sizes T=%d K=%d ff=%d top=%d", T, K, ff, top);
   IFX_REQUIRE(!paired || ff % 16 == 0, "moe_gate_up: paired weights need ff=%d to be a multiple of 16", ff);
   if (T == 0) return 0;
   const dim3 grid((unsigned)T * top, (ff + WAVES * ROWS_PER_WAVE - 1) / (WAVES * ROWS_PER_WAVE));
   hipStream_t s = (hipStream_t)stream;
   if (dtype == DT_F32)
-    hipLaunchKernelGGL(moe_gate_up_kernel<float>, grid, dim3(WAVE * WAVES), 0, s, (const float*)h, (const float*)wg, (const float*)wu, ids, (float*)act, K, ff, top, paired);
+    hipLaunchKernelGGL(moe_gate_up_kernel<float>, grid, dim3(WAVE * WAVES), 0, s, (const float*)h, (const float*)wg, (const float*)wu, ids, (float*)act, K, ff, top, paired, n_real, act_kind, limit);
   else if (dtype == DT_BF16)
-    hipLaunchKernelGGL(moe_gate_up_kernel<bf16_t>, grid, dim3(WAVE * WAVES), 0, s, (const bf16_t*)h, (const bf16_t*)wg, (const bf16_t*)wu, ids, (bf16_t*)act, K, ff, top, paired);
+    hipLaunchKernelGGL(moe_gate_up_kernel<bf16_t>, grid, dim3(WAVE * WAVES), 0, s, (const bf16_t*)h, (const bf16_t*)wg, (const bf16_t*)wu, ids, (bf16_t*)act, K, ff, top, paired, n_real, act_kind, limit);
   else IFX_FAIL("moe_gate_up: unknown dtype %d", dtype);
   IFX_LAUNCH_CHECK();
 }
 
 extern "C" int ifx_moe_down(const void* act, const void* wd, const int* ids, const float* weights, void* out, int dtype, int T,
-                            int N, int ff, int top, void* stream) {
+                            int N, int ff, int top, int n_real, const void* h, void* stream) {
   IFX_REQUIRE(T >= 0 && N > 0 && ff > 0 && top > 0, "moe_down: bad sizes T=%d N=%d ff=%d top=%d", T, N, ff, top);
+  IFX_REQUIRE(h != nullptr, "moe_down: the rows themselves are needed (identity experts read them)");
   if (T == 0) return 0;
   const dim3 grid(T, (N + WAVES * ROWS_PER_WAVE - 1) / (WAVES * ROWS_PER_WAVE));
   hipStream_t s = (hipStream_t)stream;
   if (dtype == DT_F32)
-    hipLaunchKernelGGL(moe_down_kernel<float>, grid, dim3(WAVE * WAVES), 0, s, (const float*)act, (const float*)wd, ids, weights, (float*)out, N, ff, top);
+    hipLaunchKernelGGL(moe_down_kernel<float>, grid, dim3(WAVE * WAVES), 0, s, (const float*)act, (const float*)wd, ids, weights, (float*)out, N, ff, top, n_real, (const float*)h);
   else if (dtype == DT_BF16)
-    hipLaunchKernelGGL(moe_down_kernel<bf16_t>, grid, dim3(WAVE * WAVES), 0, s, (const bf16_t*)act, (const bf16_t*)wd, ids, weights, (bf16_t*)out, N, ff, top);
+    hipLaunchKernelGGL(moe_down_kernel<bf16_t>, grid, dim3(WAVE * WAVES), 0, s, (const bf16_t*)act, (const bf16_t*)wd, ids, weights, (bf16_t*)out, N, ff, top, n_real, (const bf16_t*)h);
   else IFX_FAIL("moe_down: unknown dtype %d", dtype);
   IFX_LAUNCH_CHECK();
 }

@@ -5,6 +5,8 @@
 //   gated_add      out[t, c] = sum_slices base[.][t, c] + sigmoid(h[t] . w) * extra[t, c]: a branch that every row takes,
 //                  weighted by one number per row, added to the sum of the other branches
 //   scale_softcap  x <- cap * tanh(x * scale / cap) in place on float rows (cap 0: x <- x * scale)
+//   stream_add     x[t, c] <- x[t, c] + rows[t, c] + vec[c] in place on the float stream: what a pass of a looped span of
+//                  layers feeds into the stream before its first layer (either operand may be absent)
 // All arithmetic is float.
 #include "common.h"
 
@@ -171,5 +173,24 @@ extern "C" int ifx_scale_softcap(float* x, long long n, float scale, float cap, 
   IFX_REQUIRE(n >= 0 && cap >= 0.f, "scale_softcap: n=%lld cap=%g", n, (double)cap);
   if (n == 0) return 0;
   hipLaunchKernelGGL(scale_softcap_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, x, (size_t)n, scale, cap);
+  IFX_LAUNCH_CHECK();
+}
+
+// x [T][H] float, rows [T][H] float or null, vec [H] of any type or null
+__global__ __launch_bounds__(256) void stream_add_kernel(float* __restrict__ x, const float* __restrict__ rows, const void* __restrict__ vec,
+                                                         int vec_dtype, int H, size_t n) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  float v = x[i];
+  if (rows) v += rows[i];
+  if (vec) v += load_dyn(vec, vec_dtype, i % H);
+  x[i] = v;
+}
+
+extern "C" int ifx_stream_add(float* x, const float* rows, const void* vec, int vec_dtype, int T, int H, void* stream) {
+  IFX_REQUIRE(T >= 0 && H > 0, "stream_add: bad sizes T=%d H=%d", T, H);
+  if (T == 0 || (!rows && !vec)) return 0;
+  const size_t n = (size_t)T * H;
+  hipLaunchKernelGGL(stream_add_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, x, rows, vec, vec_dtype, H, n);
   IFX_LAUNCH_CHECK();
 }

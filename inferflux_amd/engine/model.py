@@ -35,6 +35,7 @@ class Model:
         H = plan.hidden_size
         self.embedding = build_part("embedding", plan.embedding, hidden_size=H)
         self.blocks = [build_part("block", l.block, layer=l, hidden_size=H) for l in plan.layers]
+        self.injections = [build_part("injection", spec, hidden_size=H) for spec in plan.injections]
         self.final_norm = build_part("norm", plan.final_norm, hidden_size=H)
         self.head = build_part("head", plan.lm_head, hidden_size=H)
         self.dtype: Optional[torch.dtype] = None
@@ -45,6 +46,8 @@ class Model:
         yield from _walk(self.embedding)
         for b in self.blocks:
             yield from _walk(b)
+        for j in self.injections:
+            yield from _walk(j)
         yield from _walk(self.final_norm)
         yield from _walk(self.head)
 
@@ -104,18 +107,26 @@ class Model:
         schedule = self.plan.schedule
         pending = None
         first_norm = self.blocks[schedule[0].layer].entry_norm() if schedule else None
+        if schedule and schedule[0].before is not None:
+            first_norm = None           # (rows prepared for the first norm would not know what is fed into the stream before it)
         if first_norm is not None and getattr(self.embedding, "prepares_norm_rows", False):
             residual = self.embedding.forward(ctx, norm=first_norm)     # (an embedding that can do so prepares the first norm's rows)
             if isinstance(residual, tuple):
                 residual, pending = residual
         else:
             residual = self.embedding.forward(ctx)
+        # the embedding's output as it is now, where something feeds it into the stream again later (the stream changes in place)
+        embedded = residual.clone() if any(j.needs_embedding for j in self.injections) else None
         if t is not None:
             t.mark("embed")
         for i, e in enumerate(schedule):
             block = self.blocks[e.layer]
+            if e.before is not None:
+                self.injections[e.before].forward(residual, ctx, embedded)
             # a block that can hand on rows prepared for the next block's first norm is told that norm
-            if i + 1 < len(schedule):
+            if i + 1 < len(schedule) and schedule[i + 1].before is not None:
+                following = None        # (the stream changes before that norm reads it)
+            elif i + 1 < len(schedule):
                 following = self.blocks[schedule[i + 1].layer].entry_norm()
             else:       # the last block may prepare the final norm's rows where the head takes every row of the step
                 following = self.final_norm if ctx.all_rows_wanted else None

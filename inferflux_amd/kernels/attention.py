@@ -224,21 +224,24 @@ def row_launch_shape(n_rows: int, n_kv_heads: int, max_kv: int, max_waves: int =
 
 
 def paged_attention(q: torch.Tensor, cache, ctx, window: Optional[int], scale: float, keep_first: int = 0,
-                    sink: Optional[float] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    sink: Optional[float] = None, gate: Optional[torch.Tensor] = None,
+                    sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """q [T, nH, d] of this step's rows against ``cache`` (a LayerCache); returns [T, nH*d].  ``keep_first``: the first
     positions a windowed query sees beside its window; ``sink``: the score of a key without value in the softmax's
-    denominator (None: none); ``gate`` float32 [T, nH]: a factor on every head's output."""
+    denominator (None: none), ``sinks`` float32 [nH]: such a score for every head (the plain kernel's); ``gate`` float32
+    [T, nH]: a factor on every head's output."""
     T, nH, d = q.shape
     table = ctx.block_table(cache.group)
     keep_first = int(keep_first or 0) if window else 0
-    extras = keep_first > 0 or sink is not None or gate is not None
-    if not ops.mfma_attention_supported(q.dtype, d, cache.page_size) or cache.v.shape[2] != d:
+    extras = keep_first > 0 or sink is not None or gate is not None or sinks is not None
+    if sinks is not None or not ops.mfma_attention_supported(q.dtype, d, cache.page_size) or cache.v.shape[2] != d:
         # values of another width than the keys, or heads wider than a wave's registers hold: one shared kv head (attention
         # through a latent) has a matrix-core kernel of its own, everything else (32-bit, odd sizes) the plain kernel
         if not extras and ops.wide_attention_supported(q.dtype, cache.k.shape[1], d, cache.v.shape[2], cache.page_size):
             chunk, splits = ops.wide_launch_shape(T, nH, ctx.kv_bound)
             return ops.attention_wide(q, cache.k, cache.v, ctx.row_req, ctx.positions, table, window, scale, chunk, splits)
-        return ops.attention_plain(q, cache.k, cache.v, ctx.row_req, ctx.positions, table, window, scale, keep_first, sink, gate)
+        return ops.attention_plain(q, cache.k, cache.v, ctx.row_req, ctx.positions, table, window, scale, keep_first, sink, gate,
+                                   sinks=sinks)
     n_kv = cache.k.shape[1]
     # Two query tiles per wave (128 rows per workgroup) read every key and value from LDS half as often.
     tiled = ctx.h_q_len >= TILE_MIN

@@ -26,6 +26,7 @@ _DT = {torch.float32: DT_F32, torch.bfloat16: DT_BF16}
 
 ROPE_NONE, ROPE_SPLIT_HALF, ROPE_CONSECUTIVE = 0, 1, 2
 ACT_SILU, ACT_GELU_TANH = 0, 1          # gated activations of a feed-forward: act(gate) * up
+ACT_CLAMPED_SWISH = 2                   # ... and min(gate, L) sigmoid(1.702 min(gate, L)) (clamp(up, -L, L) + 1), which takes its limit L
 _GATED_EPILOGUE = {ACT_SILU: 1, ACT_GELU_TANH: 3}    # ... as the epilogue number of the streaming products
 
 # The matrix-core attention module is compiled per head size, when a model with that head size
@@ -59,6 +60,7 @@ def module_variants() -> Iterable[Tuple[str, Variant]]:
     yield ("moe", ())
     yield ("ssm", ())
     yield ("gla", ())
+    yield ("delta", ())
     yield ("hyper", ())
     yield ("rowwise", ())
     yield ("grouped_gemm", ())
@@ -269,16 +271,17 @@ def rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], slots: Optional
     return q
 
 
-def swiglu(gate_up: torch.Tensor, interleaved: bool = False, act: int = ACT_SILU) -> torch.Tensor:
+def swiglu(gate_up: torch.Tensor, interleaved: bool = False, act: int = ACT_SILU, limit: float = 0.0) -> torch.Tensor:
     """act(gate) * up [T, I] from [T, 2I] laid out [gate | up] or, interleaved, gate_0, up_0, gate_1, ...; ``act``:
-    ACT_SILU (the default) or ACT_GELU_TANH."""
+    ACT_SILU (the default), ACT_GELU_TANH, or ACT_CLAMPED_SWISH with its ``limit`` L: g = min(gate, L),
+    u = clamp(up, -L, L), g sigmoid(1.702 g) (u + 1)."""
     _check(gate_up, "gate_up", (None, None))
     T, two_i = gate_up.shape
     if two_i % 2:
         raise KernelError("swiglu: odd width")
     out = torch.empty((T, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
-    _call(load_module("core"), "ifx_swiglu", (P, P, I, I, I, I, I, P),
-          gate_up.data_ptr(), out.data_ptr(), _dt(gate_up), T, two_i // 2, 1 if interleaved else 0, int(act), _stream())
+    _call(load_module("core"), "ifx_swiglu", (P, P, I, I, I, I, I, F, P),
+          gate_up.data_ptr(), out.data_ptr(), _dt(gate_up), T, two_i // 2, 1 if interleaved else 0, int(act), float(limit), _stream())
     return out
 
 
@@ -410,12 +413,14 @@ ROUTE_FUSED_MAX_ROWS = 16       # rows up to which the router's kernel forms the
 
 
 def moe_route(h: torch.Tensor, router, top: int, groups: int = 1, keep_groups: int = 1, group_top: int = 2,
-              softmax: bool = False, renormalize: bool = False, scale: float = 1.0, bias: Optional[torch.Tensor] = None):
+              softmax: bool = False, renormalize: bool = False, scale: float = 1.0, bias: Optional[torch.Tensor] = None,
+              choice_bias: Optional[torch.Tensor] = None):
     """The router of a mixture of experts, in float: scores of ``router`` [E, K] (a tensor or a ``LinearWeight``) times the
     rows of ``h`` [T, K] through a sigmoid (or a softmax over the experts), the ``top`` highest among the experts of the best
     ``keep_groups`` of ``groups`` equal groups of neighbours (a group scores the sum of its ``group_top`` highest).  Returns
     (ids int32 [T, top], weights float32 [T, top]): the chosen scores, divided by their sum with ``renormalize``, times
-    ``scale``.  ``bias`` float32 [E] is added to the logits before anything else.  Up to ``ROUTE_FUSED_MAX_ROWS`` rows the kernel forms the logits itself; more rows in bfloat16 get them from
+    ``scale``.  ``bias`` float32 [E] is added to the logits before anything else; ``choice_bias`` float32 [E] is added to the
+    scores for the choice alone (the weights stay the scores themselves).  Up to ``ROUTE_FUSED_MAX_ROWS`` rows the kernel forms the logits itself; more rows in bfloat16 get them from
     ``linear`` with float32 sums and output."""
     _check(h, "h", (None, None))
     T, K = h.shape
@@ -428,9 +433,11 @@ def moe_route(h: torch.Tensor, router, top: int, groups: int = 1, keep_groups: i
     weights = torch.empty((T, top), dtype=torch.float32, device=h.device)
     if bias is not None:
         _check(bias, "bias", (E,), torch.float32)
-    _call(load_module("moe"), "ifx_moe_route", (P, P, I, P, P, P, I, I, I, I, I, I, I, I, I, F, P, P),
+    if choice_bias is not None:
+        _check(choice_bias, "choice_bias", (E,), torch.float32)
+    _call(load_module("moe"), "ifx_moe_route", (P, P, I, P, P, P, I, I, I, I, I, I, I, I, I, F, P, P, P),
           h.data_ptr(), rows.data_ptr(), _dt(h), _ptr(z), ids.data_ptr(), weights.data_ptr(), T, K, E, top, groups, keep_groups,
-          group_top, 1 if softmax else 0, 1 if renormalize else 0, float(scale), _ptr(bias), _stream())
+          group_top, 1 if softmax else 0, 1 if renormalize else 0, float(scale), _ptr(bias), _ptr(choice_bias), _stream())
     return ids, weights
 
 
@@ -445,10 +452,11 @@ def pair_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
 
 
 def moe_experts(h: torch.Tensor, gate: torch.Tensor, up: Optional[torch.Tensor], down: torch.Tensor, ids: torch.Tensor,
-                weights: torch.Tensor) -> torch.Tensor:
-    """sum_j weights[t, j] * down[e] (silu(gate[e] h_t) * (up[e] h_t)), e = ids[t, j], row by row: every (row, choice)
+                weights: torch.Tensor, act: int = ACT_SILU, limit: float = 0.0, n_identity: int = 0) -> torch.Tensor:
+    """sum_j weights[t, j] * down[e] (act(gate[e] h_t, up[e] h_t)), e = ids[t, j], row by row: every (row, choice)
     streams its expert's weights (``gate`` / ``up`` [E, ff, K], or ``gate`` [E, 2 ff, K] from ``pair_gate_up`` and ``up``
-    None; ``down`` [E, N, ff]; all in h's type).  Returns [T, N]."""
+    None; ``down`` [E, N, ff]; all in h's type).  With ``n_identity`` an id from E upwards names an identity expert, whose
+    output is the row itself (N = K then).  ``act``: ACT_SILU, ACT_GELU_TANH, or ACT_CLAMPED_SWISH with its ``limit``.  Returns [T, N]."""
     _check(h, "h", (None, None))
     T, K = h.shape
     paired = up is None
@@ -461,13 +469,16 @@ def moe_experts(h: torch.Tensor, gate: torch.Tensor, up: Optional[torch.Tensor],
     top = ids.shape[1]
     _check(ids, "ids", (T, top), torch.int32)
     _check(weights, "weights", (T, top), torch.float32)
+    if n_identity and N != K:
+        raise KernelError(f"moe_experts: identity experts hand back the row itself, so N={N} must equal K={K}")
     mod = load_module("moe")
-    act = torch.empty((T, top, ff), dtype=h.dtype, device=h.device)
-    _call(mod, "ifx_moe_gate_up", (P, P, P, P, P, I, I, I, I, I, I, P),
-          h.data_ptr(), gate.data_ptr(), _ptr(up), ids.data_ptr(), act.data_ptr(), _dt(h), T, K, ff, top, 1 if paired else 0, _stream())
+    a = torch.empty((T, top, ff), dtype=h.dtype, device=h.device)
+    _call(mod, "ifx_moe_gate_up", (P, P, P, P, P, I, I, I, I, I, I, I, I, F, P),
+          h.data_ptr(), gate.data_ptr(), _ptr(up), ids.data_ptr(), a.data_ptr(), _dt(h), T, K, ff, top, 1 if paired else 0, E,
+          int(act), float(limit), _stream())
     out = torch.empty((T, N), dtype=h.dtype, device=h.device)
-    _call(mod, "ifx_moe_down", (P, P, P, P, P, I, I, I, I, I, P),
-          act.data_ptr(), down.data_ptr(), ids.data_ptr(), weights.data_ptr(), out.data_ptr(), _dt(h), T, N, ff, top, _stream())
+    _call(mod, "ifx_moe_down", (P, P, P, P, P, I, I, I, I, I, I, P, P),
+          a.data_ptr(), down.data_ptr(), ids.data_ptr(), weights.data_ptr(), out.data_ptr(), _dt(h), T, N, ff, top, E, h.data_ptr(), _stream())
     return out
 
 
@@ -483,11 +494,12 @@ def grouped_takes(dtype: torch.dtype, K: int, ff: int) -> bool:
 
 
 def moe_experts_grouped(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, ids: torch.Tensor,
-                        weights: torch.Tensor) -> "SliceSums":
+                        weights: torch.Tensor, act: int = ACT_SILU, limit: float = 0.0, n_identity: int = 0) -> "SliceSums":
     """The same sum for steps of many rows, on the matrix cores: the (row, choice) items are ordered by expert on the
     device and every expert's weights meet tiles of its items (bfloat16; ``gate_up`` from ``pair_gate_up``).  Returns the
     choices' weighted outputs as ``SliceSums`` [top, T, N] (float32), which the kernel that adds them to the stream sums
-    in the order of the choices."""
+    in the order of the choices.  ``n_identity``: ids from E up to E + n_identity name identity experts, whose output is
+    the row itself (N = K then); ``act`` and ``limit`` as for ``moe_experts``."""
     _check(h, "h", (None, None), torch.bfloat16)
     T, K = h.shape
     _check(gate_up, "gate_up", (None, None, K), torch.bfloat16)
@@ -499,7 +511,10 @@ def moe_experts_grouped(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tens
     if not grouped_takes(h.dtype, K, ff):
         raise KernelError(f"moe_experts_grouped: K={K} must be a multiple of 8 and ff={ff} of 16")
     mod = load_module("grouped_gemm")
+    if n_identity and N != K:
+        raise KernelError(f"moe_experts_grouped: identity experts hand back the row itself, so N={N} must equal K={K}")
     n_items = T * top
+    n_real, E = E, E + int(n_identity)
     tile_items = grouped_tile_items(n_items, E)
     max_tiles = -(-n_items // tile_items) + E          # every expert may end on a tile that is not full
     lists = torch.empty((n_items + 3 * max_tiles + 1,), dtype=torch.int32, device=h.device)
@@ -507,14 +522,14 @@ def moe_experts_grouped(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tens
                                lists[n_items + 2 * max_tiles:n_items + 3 * max_tiles], lists[n_items + 3 * max_tiles:])
     _call(mod, "ifx_moe_sort", (P, I, I, I, P, P, P, P, P, P), ids.data_ptr(), n_items, E, tile_items, sorted_.data_ptr(), te.data_ptr(),
           ts.data_ptr(), tc.data_ptr(), nt.data_ptr(), _stream())
-    act = torch.empty((n_items, ff), dtype=torch.bfloat16, device=h.device)
-    _call(mod, "ifx_moe_gate_up_grouped", (P, P, P, P, P, P, P, P, I, I, I, I, I, P),
-          h.data_ptr(), gate_up.data_ptr(), act.data_ptr(), sorted_.data_ptr(), te.data_ptr(), ts.data_ptr(), tc.data_ptr(),
-          nt.data_ptr(), max_tiles, tile_items, K, ff, top, _stream())
+    a = torch.empty((n_items, ff), dtype=torch.bfloat16, device=h.device)
+    _call(mod, "ifx_moe_gate_up_grouped", (P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P),
+          h.data_ptr(), gate_up.data_ptr(), a.data_ptr(), sorted_.data_ptr(), te.data_ptr(), ts.data_ptr(), tc.data_ptr(),
+          nt.data_ptr(), max_tiles, tile_items, K, ff, top, n_real, int(act), float(limit), _stream())
     parts = torch.empty((top, T, N), dtype=torch.float32, device=h.device)
-    _call(mod, "ifx_moe_down_grouped", (P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, P),
-          act.data_ptr(), down.data_ptr(), parts.data_ptr(), weights.data_ptr(), sorted_.data_ptr(), te.data_ptr(), ts.data_ptr(),
-          tc.data_ptr(), nt.data_ptr(), max_tiles, tile_items, T, N, ff, top, _stream())
+    _call(mod, "ifx_moe_down_grouped", (P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, P),
+          a.data_ptr(), down.data_ptr(), parts.data_ptr(), weights.data_ptr(), sorted_.data_ptr(), te.data_ptr(), ts.data_ptr(),
+          tc.data_ptr(), nt.data_ptr(), max_tiles, tile_items, T, N, ff, top, n_real, h.data_ptr(), _stream())
     return SliceSums(parts, torch.bfloat16)
 
 
@@ -1035,8 +1050,9 @@ def _small_m_kernel(M: int, N: int, K: int, has_tiled: bool = False) -> Optional
     return None
 
 
-def linear_swiglu(x: torch.Tensor, weight_pairs, act: int = ACT_SILU) -> torch.Tensor:
-    """act(x Wg^T) * (x Wu^T) (``act``: ACT_SILU or ACT_GELU_TANH) where ``weight_pairs`` [2I, K] (a tensor or a
+def linear_swiglu(x: torch.Tensor, weight_pairs, act: int = ACT_SILU, limit: float = 0.0) -> torch.Tensor:
+    """act(x Wg^T) * (x Wu^T) (``act``: ACT_SILU, ACT_GELU_TANH, or ACT_CLAMPED_SWISH with its ``limit``, which is applied by
+    a kernel of its own after the product whatever the number of rows) where ``weight_pairs`` [2I, K] (a tensor or a
     ``LinearWeight``) alternates the rows of Wg and Wu.  For few rows the activation is the product's epilogue; otherwise a second kernel
     applies it."""
     M, K = x.shape
@@ -1046,6 +1062,8 @@ def linear_swiglu(x: torch.Tensor, weight_pairs, act: int = ACT_SILU) -> torch.T
                               else (weight_pairs, None, 16))
     if isinstance(weight_pairs, LinearWeight) and weight_pairs.order is not None:
         raise KernelError("linear_swiglu: a tile order is not supported for gate/up pairs")
+    if act == ACT_CLAMPED_SWISH:
+        return swiglu(linear(x, weight_pairs), interleaved=True, act=act, limit=limit)
     if rows.dtype == torch.bfloat16 and x.dtype == torch.bfloat16:
         kind = _small_m_kernel(M, rows.shape[0], K, tiled is not None)
         if kind == "skinny":
@@ -1061,13 +1079,24 @@ def linear_swiglu(x: torch.Tensor, weight_pairs, act: int = ACT_SILU) -> torch.T
 def attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_req: torch.Tensor,
                     positions: torch.Tensor, block_table: torch.Tensor, window: Optional[int],
                     scale: float, keep_first: int = 0, sink: Optional[float] = None,
-                    gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    gate: Optional[torch.Tensor] = None, sinks: Optional[torch.Tensor] = None, chunk: Optional[int] = None,
+                    differential: Optional[Tuple[float, float, float]] = None) -> torch.Tensor:
     """Causal (optionally windowed) attention of q [T, nH, d] over the paged cache (K [pages, nKV, page, d],
     V [pages, nKV, dv, page]; dv may differ from d); returns [T, nH*dv].  ``keep_first``: a windowed query also sees
     the first so many positions of its request; ``sink``: the score of a key without value that is added to the
-    softmax's denominator (None: no such key); ``gate`` float32 [T, nH]: a factor on every head's output."""
+    softmax's denominator (None: no such key), ``sinks`` float32 [nH]: such a score for every head; ``gate`` float32
+    [T, nH]: a factor on every head's output; ``chunk``: a query sees only keys of its own block of that many positions,
+    counted from the sequence's start.  ``differential`` (lambda, out_scale, eps): q and the keys hold two vectors of
+    d / 2 elements per head, each pair a softmax map of its own over the same values; a head's output is map 1 minus
+    lambda times map 2, divided by its root mean square (eps inside the root), times out_scale."""
     _check(q, "q", (None, None, None))
     T, nH, d = q.shape
+    maps = 2 if differential is not None else 1
+    if d % maps:
+        raise KernelError(f"attention_plain: two maps need an even row, got {d}")
+    lam, out_scale, norm_eps = differential if differential is not None else (0.0, 1.0, 0.0)
+    if sinks is not None:
+        _check(sinks, "sinks", (nH,), torch.float32)
     _check(k_cache, "k_cache", (None, None, None, d), q.dtype)
     n_pages, nKV, page_size, _ = k_cache.shape
     _check(v_cache, "v_cache", (n_pages, nKV, None, page_size), q.dtype)
@@ -1078,11 +1107,83 @@ def attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     if gate is not None:
         _check(gate, "gate", (T, nH), torch.float32)
     out = torch.empty((T, nH * dv), dtype=q.dtype, device=q.device)
-    _call(load_module("attn_plain"), "ifx_attn_plain", (P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, I, F, P, P),
+    _call(load_module("attn_plain"), "ifx_attn_plain", (P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, I, I, F, P, P, I, I, F, F, F, P),
           q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _dt(q), row_req.data_ptr(),
-          positions.data_ptr(), block_table.data_ptr(), block_table.shape[1], T, nH, nKV, d, dv, page_size,
-          int(window or 0), float(scale), int(keep_first or 0), 0 if sink is None else 1, float(sink or 0.0), _ptr(gate), _stream())
+          positions.data_ptr(), block_table.data_ptr(), block_table.shape[1], T, nH, nKV, d // maps, dv, page_size,
+          int(window or 0), float(scale), int(keep_first or 0), 0 if sink is None else 1, float(sink or 0.0), _ptr(gate),
+          _ptr(sinks), int(chunk or 0), maps, float(lam), float(out_scale), float(norm_eps), _stream())
     return out
+
+
+# ----------------------------------------------------------------------------------------
+DELTA_THREAD_CHANNELS = (8, 16, 32, 64)     # key channels of a column of S a thread may hold
+DELTA_MAX_PADDED_DIM, DELTA_MAX_V_DIM = 256, 512
+
+
+def delta_layout(d: int, dv: int) -> Tuple[int, int]:
+    """(channels a thread, threads a column) of the delta rule's kernel for heads of ``d`` key channels and ``dv`` values:
+    the fewest channels a thread whose columns still fit a workgroup of 1,024 threads (the threads of a column are a
+    power of two of neighbouring lanes)."""
+    for ch in DELTA_THREAD_CHANNELS:
+        ks = 1
+        while ks * ch < d:
+            ks *= 2
+        if ks <= 64 and ks * ch <= DELTA_MAX_PADDED_DIM and dv * ks <= 1024 and dv <= DELTA_MAX_V_DIM:
+            return ch, ks
+    raise KernelError(f"delta rule: heads of {d} key channels and {dv} values fit no layout of the kernel (at most "
+                      f"{DELTA_MAX_PADDED_DIM} channels, {DELTA_MAX_V_DIM} values, and columns x threads a column within 1,024)")
+
+
+def delta_state_floats(n_heads: int, d: int, dv: int) -> int:
+    ch, ks = delta_layout(d, dv)
+    return n_heads * dv * ch * ks
+
+
+def delta_rule(u: torch.Tensor, rows: torch.Tensor, cols: Tuple[int, int, int], A_log: torch.Tensor, dt_bias: torch.Tensor,
+               norm_w: torch.Tensor, eps: float, n_heads: int, n_kv_heads: int, d: int, dv: int, state: torch.Tensor,
+               state_offset: int, q_start: torch.Tensor, q_len: torch.Tensor, slots: torch.Tensor) -> torch.Tensor:
+    """The gated delta rule over a step's rows (see csrc/delta.hip).  ``u`` [T, >= 2 G d + H dv] holds per row the q heads,
+    the k heads and the v heads (after their convolution), ``rows`` [T, ld] the gate's H dv columns from ``cols[0]``, beta's
+    H from ``cols[1]`` and the decay's H from ``cols[2]``, both in the activation type.  ``A_log``, ``dt_bias`` float32 [H],
+    ``norm_w`` [dv].  A request's S lies ``state_offset`` floats into its row of ``state`` [slots, n] (float32), zero for a
+    request that starts.  Returns [T, H dv] in u's type."""
+    _check(u, "u", (None, None))
+    T, ldu = u.shape
+    _check(rows, "rows", (T, None), u.dtype)
+    ldr = rows.shape[1]
+    H, G = n_heads, n_kv_heads
+    col_g, col_b, col_a = cols
+    if ldu < 2 * G * d + H * dv or col_g + H * dv > ldr or col_b + H > ldr or col_a + H > ldr:
+        raise KernelError("delta_rule: the rows are narrower than the columns named")
+    _check(A_log, "A_log", (H,), torch.float32)
+    _check(dt_bias, "dt_bias", (H,), torch.float32)
+    _check(norm_w, "norm_w", (dv,))
+    _check(state, "state", (None, None), torch.float32)
+    R = q_start.shape[0]
+    for t, nm in ((q_start, "q_start"), (q_len, "q_len"), (slots, "slots")):
+        _check(t, nm, (R,), torch.int32)
+    ch, ks = delta_layout(d, dv)
+    if state_offset + H * dv * ch * ks > state.shape[1]:
+        raise KernelError("delta_rule: the state rows are too short")
+    out = torch.empty((T, H * dv), dtype=u.dtype, device=u.device)
+    _call(load_module("delta"), "ifx_delta_rule", (P, I, P, I, I, I, I, I, P, P, P, I, F, P, LL, LL, P, P, P, P, I, I, I, I, I, I, I, P),
+          u.data_ptr(), ldu, rows.data_ptr(), ldr, col_g, col_b, col_a, _dt(u), A_log.data_ptr(), dt_bias.data_ptr(),
+          norm_w.data_ptr(), _dt(norm_w), float(eps), state.data_ptr(), state.shape[1], int(state_offset), q_start.data_ptr(),
+          q_len.data_ptr(), slots.data_ptr(), out.data_ptr(), R, H, G, d, dv, ch, ks, _stream())
+    return out
+
+
+def stream_add(stream: torch.Tensor, rows: Optional[torch.Tensor] = None, vec: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """stream [T, H] (float32) += rows [T, H] (float32) + vec [H], in place; either operand may be None."""
+    _check(stream, "stream", (None, None), torch.float32)
+    T, H = stream.shape
+    if rows is not None:
+        _check(rows, "rows", (T, H), torch.float32)
+    if vec is not None:
+        _check(vec, "vec", (H,))
+    _call(load_module("rowwise"), "ifx_stream_add", (P, P, P, I, I, I, P), stream.data_ptr(), _ptr(rows), _ptr(vec),
+          _dt(vec) if vec is not None else 0, T, H, _stream())
+    return stream
 
 
 # ----------------------------------------------------------------------------------------

@@ -1,5 +1,5 @@
 """Parts a model is assembled from.  Importing the package registers the built-in parts."""
-from . import attention, block, embedding, ffn, gla, latent_attention, moe, norm, position, ssm  # noqa: F401
+from . import attention, block, delta, embedding, ffn, gla, injection, latent_attention, moe, norm, position, ssm  # noqa: F401
 from .base import (Block, FeedForward, LayerCache, Mixer, MixerBinding, Norm, Part, build_part,
                    register_part, registered_parts)
 from .plan import (CacheSpec, LayerSpec, ModelPlan, ParamSpec, PartSpec, ScheduleEntry, StateSpec)

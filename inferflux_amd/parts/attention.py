@@ -27,8 +27,17 @@ Optional mechanisms, each a constructor argument that is off by default:
   ``value_mix``       "source": this layer hands the step's values (as projected) on to the layers after it; "mix": this
                       layer caches v <- (1 - lambda) v + lambda v_source instead of its own, lambda a scalar tensor.  The
                       layers must agree in kv heads and value width.
+  ``chunk``           the sequence is cut into blocks of this many positions counted from its start, and a query sees only
+                      the keys of its own block: j <= i and j // chunk == i // chunk.  The cache keeps a window of ``chunk``
+                      positions (a block never reaches further back).
+  ``differential``    {"diff": c, "eps": e}: differential attention.  Every query head and kv head holds two vectors of
+                      ``head_dim`` elements, laid out one after the other; each pair is a softmax map of its own over the
+                      same values a_1, a_2, and the head's output is o = a_1 - lambda a_2 with lambda =
+                      exp(lq1 . lk1) - exp(lq2 . lk2) + c (four tensors of head_dim, one lambda for the layer), then
+                      o / sqrt(mean(o^2) + e) over the head's values, times (1 - c).  Needs a position part that leaves q
+                      and k alone.
   ``tensors``         full names of the tensors in the model file ("q", "k", "v", "o", "q_bias", "k_bias", "v_bias", "gate",
-                      "mix", "q_norm", "k_norm") where they are not ``<name>.q_proj.weight`` and so on.
+                      "mix", "q_norm", "k_norm", "lq1", "lk1", "lq2", "lk2") where they are not ``<name>.q_proj.weight`` and so on.
 """
 from __future__ import annotations
 
@@ -40,6 +49,7 @@ import torch
 from ..kernels import ops
 from ..kernels.attention import paged_attention
 from .base import Mixer, MixerBinding, build_part, register_part
+from .position import PositionEncoding
 from .ffn import concat_weights
 from .plan import CacheSpec, ParamSpec, PartSpec
 
@@ -53,16 +63,24 @@ class PagedAttention(Mixer):
                  scale: Optional[float] = None, init_std: float = 0.02, v_head_dim: Optional[int] = None,
                  keep_first: int = 0, sink: Optional[float] = None, unit_norm_eps: Optional[float] = None,
                  output_gate=False, value_mix: Optional[str] = None, tensors: Optional[Mapping[str, str]] = None,
-                 qk_norm_eps: Optional[float] = None):
+                 qk_norm_eps: Optional[float] = None, chunk: Optional[int] = None, differential: Optional[Mapping[str, float]] = None):
         """``v_head_dim``: the width of a value head where it differs from ``head_dim`` (such a layer runs on the
         kernels that take both widths: the plain attention kernel and the unfused projection path)."""
         if n_heads % n_kv_heads:
             raise ValueError(f"{name}: {n_heads} query heads are not a multiple of {n_kv_heads} kv heads")
         self.name, self.hidden_size = name, int(hidden_size)
+        self.chunk = int(chunk) if chunk else None
+        self.differential = None
+        self.map_dim = int(head_dim)                   # elements of one map's query or key
+        if differential is not None:
+            self.differential = (float(differential["diff"]), float(differential["eps"]))
+            head_dim = 2 * int(head_dim)               # to the projection, the row kernel and the cache a head is both maps' vectors
+        if v_head_dim is None and differential is not None:
+            v_head_dim = self.map_dim
         self.n_heads, self.n_kv_heads, self.head_dim = int(n_heads), int(n_kv_heads), int(head_dim)
         self.v_head_dim = int(v_head_dim) if v_head_dim else self.head_dim
         self.bias, self.window, self.init_std = bool(bias), (int(window) if window else None), init_std
-        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.map_dim)
         self.position = build_part("position", position)
         self.keep_first = max(int(keep_first or 0), 0) if self.window else 0
         self.sink = None if sink is None else float(sink)
@@ -79,11 +97,16 @@ class PagedAttention(Mixer):
         self.names = {"q": f"{name}.q_proj.weight", "k": f"{name}.k_proj.weight", "v": f"{name}.v_proj.weight",
                       "o": f"{name}.o_proj.weight", "q_bias": f"{name}.q_proj.bias", "k_bias": f"{name}.k_proj.bias",
                       "v_bias": f"{name}.v_proj.bias", "gate": f"{name}.gate.weight", "mix": f"{name}.value_mix",
-                      "q_norm": f"{name}.q_norm.weight", "k_norm": f"{name}.k_norm.weight"}
+                      "q_norm": f"{name}.q_norm.weight", "k_norm": f"{name}.k_norm.weight",
+                      "lq1": f"{name}.lambda_q1", "lk1": f"{name}.lambda_k1", "lq2": f"{name}.lambda_q2", "lk2": f"{name}.lambda_k2"}
         self.names.update(tensors or {})
         # (what the kernels fused for the plain case do not do: then the projection, the row kernel and attention run one by one)
         self._extras = (self.unit_norm_eps is not None or self.output_gate or self.value_mix is not None
-                        or self.qk_norm_eps is not None)
+                        or self.qk_norm_eps is not None or self.chunk is not None or self.differential is not None)
+        if self.differential is not None and (self.unit_norm_eps is not None or self.qk_norm_eps is not None
+                                              or self.position.kernel_args.__func__ is not PositionEncoding.kernel_args):
+            raise ValueError(f"{name}: differential attention takes no norms on q and k and a position part that leaves them alone")
+        self.lam = 0.0
         self.w_qkv = self.b_qkv = self.w_o = self._w_q = None
 
     @property
@@ -94,7 +117,10 @@ class PagedAttention(Mixer):
         return self.n_heads * self.v_head_dim if self.gate_elementwise else self.n_heads
 
     def cache_spec(self) -> CacheSpec:
-        return CacheSpec(self.n_kv_heads, self.head_dim, self.window,
+        window = self.window
+        if self.chunk is not None:             # a block's query never reads further back than the block is long
+            window = min(window, self.chunk) if window else self.chunk
+        return CacheSpec(self.n_kv_heads, self.head_dim, window,
                          self.v_head_dim if self.v_head_dim != self.head_dim else None, self.keep_first)
 
     def param_specs(self) -> Dict[str, ParamSpec]:
@@ -115,6 +141,9 @@ class PagedAttention(Mixer):
         if self.qk_norm_eps is not None:
             out[nm["q_norm"]] = ParamSpec((d,), ("ones",))
             out[nm["k_norm"]] = ParamSpec((d,), ("ones",))
+        if self.differential is not None:
+            for k in ("lq1", "lk1", "lq2", "lk2"):
+                out[nm[k]] = ParamSpec((self.map_dim,), ("normal", 0.1))
         if self.value_mix is not None:       # (the source layer's tensor is in the file too, where the file has it; nothing reads it)
             out[nm["mix"]] = ParamSpec((), ("uniform", 0.2, 0.8), optional=self.value_mix == "source")
         return out
@@ -136,6 +165,9 @@ class PagedAttention(Mixer):
             self.q_norm_w, self.k_norm_w = tensors[nm["q_norm"]], tensors[nm["k_norm"]]
             if self.q_norm_w.dtype != self.k_norm_w.dtype:
                 self.q_norm_w, self.k_norm_w = self.q_norm_w.float(), self.k_norm_w.float()
+        if self.differential is not None:      # one number for the layer, formed once in double precision
+            dot = lambda a, b: float((tensors[nm[a]].double() * tensors[nm[b]].double()).sum().item())
+            self.lam = math.exp(dot("lq1", "lk1")) - math.exp(dot("lq2", "lk2")) + self.differential[0]
         self._w_q = None
 
     def _prepare_qkv(self, weight: torch.Tensor, heads: int):
@@ -159,6 +191,11 @@ class PagedAttention(Mixer):
         return ops.linear(out, self.w_o, keep_slices=sink is not None)   # an RMS norm's kernel adds partial sums itself
 
     def _attend(self, q, cache, ctx, gate=None):
+        if self.chunk is not None or self.differential is not None:
+            # the kernel that knows blocks and two maps: one wave per (row, head), float or bfloat16 storage, float math
+            diff = None if self.differential is None else (self.lam, 1.0 - self.differential[0], self.differential[1])
+            return ops.attention_plain(q, cache.k, cache.v, ctx.row_req, ctx.positions, ctx.block_table(cache.group), self.window,
+                                       self.scale, self.keep_first, self.sink, gate, chunk=self.chunk, differential=diff)
         return paged_attention(q, cache, ctx, self.window, self.scale, self.keep_first, self.sink, gate)
 
     def _forward_extras(self, h, ctx, binding: MixerBinding, sink):

@@ -21,6 +21,10 @@ Categories and what each must provide beyond ``param_specs`` / ``load``:
   embedding forward(ctx) -> float32 stream [T, H] of the step's rows (``ctx.token_ids``, and whatever else of the
             step it needs: ``ctx.positions`` for a learned position table, ...).
   head      forward(normalised rows) -> float32 logits [R, V].
+  injection forward(residual, ctx, embedded) -> None: changes the float32 stream in place right before the layer of the
+            schedule entry that names it.  ``embedded`` is the embedding's output for the step's rows as it was before the
+            first layer (kept for the step only if some injection says ``needs_embedding``).  Whatever the block before
+            has not added to the stream yet is added later as before; an addition commutes.
 
 A norm's kernel can be saved for steps of few rows, where a launch costs as much as the work.  This is
 optional for every part; one that declares nothing is run as above.
@@ -50,7 +54,7 @@ import torch
 from .plan import CacheSpec, ParamSpec, PartSpec, StateSpec
 
 _REGISTRY: Dict[str, Dict[str, Callable]] = {}
-CATEGORIES = ("norm", "position", "mixer", "ffn", "block", "embedding", "head")
+CATEGORIES = ("norm", "position", "mixer", "ffn", "block", "embedding", "head", "injection")
 
 
 def register_part(category: str, name: str):
@@ -172,6 +176,13 @@ class Norm(Part):
 
     def forward(self, residual: torch.Tensor, delta: Optional[torch.Tensor], out_dtype: torch.dtype,
                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Injection(Part):
+    needs_embedding = False
+
+    def forward(self, residual: torch.Tensor, ctx, embedded: Optional[torch.Tensor]) -> None:
         raise NotImplementedError
 
 

@@ -1,5 +1,6 @@
 """Gated feed-forward: down( act(gate(x)) * up(x) ), no biases; act is silu ("SwiGLU", the default) or the tanh form
-of gelu, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))).
+of gelu, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))).  "clamped_swish" with its ``limit`` L is another form of the
+inner part: g = min(gate(x), L), u = clamp(up(x), -L, L), down( g sigmoid(1.702 g) (u + 1) ).
 
 g = h Wg^T, u = h Wu^T, a = g / (1 + exp(-g)) * u in float, delta = a Wd^T
 (runtime/backends/cuda/native/transformer_forward.cu:2383-2419, 2487-2494, 2528-2547;
@@ -28,6 +29,7 @@ def concat_weights(parts):
 
 
 ACTIVATIONS = {"silu": ops.ACT_SILU, "gelu_tanh": ops.ACT_GELU_TANH}
+GATED_ACTIVATIONS = {**ACTIVATIONS, "clamped_swish": ops.ACT_CLAMPED_SWISH}      # (the last one takes a limit)
 
 
 @register_part("ffn", "gated_ffn")
@@ -36,14 +38,17 @@ class SwiGLU(FeedForward):
     graph_safe = True
 
     def __init__(self, name: str, hidden_size: int, intermediate_size: int, init_std: float = 0.02,
-                 activation: str = "silu", tensors: Optional[Mapping[str, str]] = None):
-        """``activation``: "silu" or "gelu_tanh".  ``tensors``: the full names of "gate", "up" and "down" in the model
-        file where they are not ``<name>.gate_proj.weight`` and so on."""
+                 activation: str = "silu", tensors: Optional[Mapping[str, str]] = None, limit: Optional[float] = None):
+        """``activation``: "silu", "gelu_tanh" or "clamped_swish" (with its ``limit``).  ``tensors``: the full names of
+        "gate", "up" and "down" in the model file where they are not ``<name>.gate_proj.weight`` and so on."""
         self.name, self.hidden_size, self.intermediate_size = name, int(hidden_size), int(intermediate_size)
         self.init_std = init_std
-        if activation not in ACTIVATIONS:
-            raise ValueError(f"{name}: activation '{activation}' unknown (one of {sorted(ACTIVATIONS)})")
-        self.activation, self.act = activation, ACTIVATIONS[activation]
+        if activation not in GATED_ACTIVATIONS:
+            raise ValueError(f"{name}: activation '{activation}' unknown (one of {sorted(GATED_ACTIVATIONS)})")
+        self.activation, self.act = activation, GATED_ACTIVATIONS[activation]
+        self.limit = float(limit) if limit is not None else 0.0
+        if (self.act == ops.ACT_CLAMPED_SWISH) != (self.limit > 0):
+            raise ValueError(f"{name}: the activation '{activation}' and a limit of {limit} do not go together")
         self.names = {k: f"{name}.{k}_proj.weight" for k in ("gate", "up", "down")}
         self.names.update(tensors or {})
         self.w_gate_up = None
@@ -71,7 +76,7 @@ class SwiGLU(FeedForward):
         return ops.takes_scaled_rows(n_rows, self.w_gate_up)
 
     def forward(self, h, ctx, sink=None):
-        a = ops.linear_swiglu(h, self.w_gate_up, self.act)
+        a = ops.linear_swiglu(h, self.w_gate_up, self.act, self.limit)
         if ctx.timer is not None:
             ctx.timer.mark("ffn.gate_up")
         if sink is not None and ops.adds_into_stream(a.shape[0], self.w_down, sink.norm_weight):

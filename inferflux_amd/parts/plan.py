@@ -4,7 +4,10 @@ A ``ModelPlan`` is produced from a typed config by the architecture's plan build
 is all the generic model needs: it names parts by their registry name with their sizes
 and constants as arguments, layer by layer, so layers of one model may differ in mixer,
 feed-forward, norm or window.  The run order (``schedule``) is a list too: it may name a
-layer twice, and an entry may read the cache that another entry writes.
+layer twice, and an entry may read the cache that another entry writes.  An entry may also name
+something that is fed into the stream right before its layer runs (``before``: an index into the
+plan's ``injections``), which is how a span of layers that runs several times is given its pass's
+input.
 """
 from __future__ import annotations
 
@@ -49,10 +52,12 @@ class ScheduleEntry:
 
     ``layer`` indexes ``ModelPlan.layers``.  ``cache_from`` is None when the entry's mixer
     owns a cache of its own, or the index of an earlier schedule entry whose cache this
-    entry's mixer reads without writing.
+    entry's mixer reads without writing.  ``before`` is None, or the index of the injection (``ModelPlan.injections``)
+    that changes the stream right before this entry's layer.
     """
     layer: int
     cache_from: Optional[int] = None
+    before: Optional[int] = None
 
 
 @dataclasses.dataclass(frozen=True)
@@ -66,6 +71,7 @@ class ModelPlan:
     final_norm: PartSpec
     lm_head: PartSpec
     eos_token_ids: Tuple[int, ...] = ()      # every token id that ends a request (a model may name several)
+    injections: Tuple[PartSpec, ...] = ()    # parts of category "injection" that schedule entries name in ``before``
 
     def validate(self) -> None:
         if not self.layers:
@@ -73,6 +79,8 @@ class ModelPlan:
         for i, e in enumerate(self.schedule):
             if not (0 <= e.layer < len(self.layers)):
                 raise ValueError(f"schedule[{i}] names layer {e.layer}, plan has {len(self.layers)}")
+            if e.before is not None and not (0 <= e.before < len(self.injections)):
+                raise ValueError(f"schedule[{i}].before={e.before}, plan has {len(self.injections)} injections")
             if e.cache_from is not None:
                 if not (0 <= e.cache_from < i):
                     raise ValueError(f"schedule[{i}].cache_from={e.cache_from} must name an earlier entry")
