@@ -31,15 +31,16 @@ def softplus(z):
 
 # ---- masks ------------------------------------------------------------------------------------------------------------
 def chunk_mask(T, size):
-    """[T, T] True where query i sees key j: j <= i and both in the same block of ``size`` positions counted from 0."""
+    """[T, T] True where query i sees key j: j <= i and both in the same block of ``size`` positions counted from 0 (None:
+    every j <= i)."""
     i, j = np.arange(T)[:, None], np.arange(T)[None, :]
-    return (j <= i) & (i // size == j // size)
+    return (j <= i) if size is None else (j <= i) & (i // size == j // size)
 
 
 def window_mask(T, size):
-    """[T, T] True where query i sees key j: 0 <= i - j < size."""
+    """[T, T] True where query i sees key j: 0 <= i - j < size (None: every j <= i)."""
     i, j = np.arange(T)[:, None], np.arange(T)[None, :]
-    return (j <= i) & (i - j < size)
+    return (j <= i) if size is None else (j <= i) & (i - j < size)
 
 
 def masked_softmax(s, mask, sink=None):
@@ -56,15 +57,19 @@ def masked_softmax(s, mask, sink=None):
 
 
 # ---- differential attention -------------------------------------------------------------------------------------------
+def _size(m):
+    return (m.get("mask") or {}).get("size")
+
+
 def differential_attention(h, W, p, m, eps):
     """Two softmax maps per head over the same values, the second subtracted lambda times; chunked mask; no positions."""
     T = h.shape[0]
-    H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    H, G, d, dv = m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m.get("vdim", m["dim"])
     q = (h @ W[p + ".q"].T + W[p + ".q.b"]).reshape(T, H, 2, d)
     k = (h @ W[p + ".k"].T + W[p + ".k.b"]).reshape(T, G, 2, d)
     v = (h @ W[p + ".v"].T + W[p + ".v.b"]).reshape(T, G, dv)
     lam = math.exp(float(np.sum(W[p + ".lq1"] * W[p + ".lk1"]))) - math.exp(float(np.sum(W[p + ".lq2"] * W[p + ".lk2"]))) + m["diff"]
-    mask = chunk_mask(T, m["mask"]["size"])
+    mask = chunk_mask(T, _size(m))
     out = np.zeros((T, H, dv))
     for hd in range(H):
         g = hd // (H // G)
@@ -87,9 +92,21 @@ def unit(x):
     return x / np.sqrt(np.sum(x * x, axis=-1, keepdims=True) + 1e-6)
 
 
+def delta_recurrence(q, k, v, beta, decay):
+    """One head: q, k [T, d], v [T, dv], beta, decay [T].  S <- decay S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q."""
+    T, d = q.shape
+    S, out = np.zeros((d, v.shape[1])), np.zeros_like(v)
+    for t in range(T):
+        S = decay[t] * S
+        u = beta[t] * (v[t] - S.T @ k[t])
+        S = S + np.outer(k[t], u)
+        out[t] = S.T @ q[t]
+    return out
+
+
 def gated_delta(h, W, p, m, eps):
     T = h.shape[0]
-    H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    H, G, d, dv = m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m.get("vdim", m["dim"])
     q = silu(causal_conv(h @ W[p + ".q"].T, W[p + ".q.conv"])).reshape(T, G, d)
     k = silu(causal_conv(h @ W[p + ".k"].T, W[p + ".k.conv"])).reshape(T, G, d)
     v = silu(causal_conv(h @ W[p + ".v"].T, W[p + ".v.conv"])).reshape(T, H, dv)
@@ -100,12 +117,7 @@ def gated_delta(h, W, p, m, eps):
     out = np.zeros((T, H, dv))
     for hd in range(H):
         g = hd // (H // G)
-        S = np.zeros((d, dv))
-        for t in range(T):
-            S = decay[t, hd] * S
-            u = beta[t, hd] * (v[t, hd] - S.T @ k[t, g])
-            S = S + np.outer(k[t, g], u)
-            out[t, hd] = S.T @ q[t, g]
+        out[:, hd] = delta_recurrence(q[:, g], k[:, g], v[:, hd], beta[:, hd], decay[:, hd])
     out = rms_norm(out, W[p + ".norm"], eps) * gate
     return out.reshape(T, H * dv) @ W[p + ".o"].T
 
@@ -126,15 +138,16 @@ def rotate_pairs(x, positions, dims, base):
 
 def latent_attention(h, W, p, m, eps, positions):
     T = h.shape[0]
-    H, d, r, dv, rank = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
+    H, d, r, dv, rank = m["heads"], m["dim"], m["rot_dim"], m.get("vdim", m["dim"]), m["kv_rank"]
+    dims = m["rot"].get("dims", r)
     q = (h @ W[p + ".q"].T).reshape(T, H, d + r)
     down = h @ W[p + ".dkv"].T
     c = rms_norm(down[:, :rank], W[p + ".dkv.norm"], eps)
-    k_rot = rotate_pairs(down[:, rank:], positions, m["rot"]["dims"], m["rot"]["base"])      # [T, r], one for all heads
-    q_rot = rotate_pairs(q[:, :, d:], positions, m["rot"]["dims"], m["rot"]["base"])
+    k_rot = rotate_pairs(down[:, rank:], positions, dims, m["rot"]["base"])      # [T, r], one for all heads
+    q_rot = rotate_pairs(q[:, :, d:], positions, dims, m["rot"]["base"])
     k_plain = (c @ W[p + ".uk"].T).reshape(T, H, d)
     v = (c @ W[p + ".uv"].T).reshape(T, H, dv)
-    mask = window_mask(T, m["mask"]["size"])
+    mask = window_mask(T, _size(m))
     out = np.zeros((T, H, dv))
     for hd in range(H):
         s = (q[:, hd, :d] @ k_plain[:, hd].T + q_rot[:, hd] @ k_rot.T) * m["scale"]
@@ -156,7 +169,7 @@ def route(h, W, p, r):
     s = s / s.sum(axis=-1, keepdims=True)
     choice = s + W[p + ".correction"]
     ids = np.argsort(-choice, axis=-1, kind="stable")[:, :r["top"]]
-    return ids, np.take_along_axis(s, ids, axis=-1) * r["scale"]
+    return ids, np.take_along_axis(s, ids, axis=-1) * r.get("scale", 1.0)
 
 
 def moe(h, W, p, m):
@@ -213,3 +226,11 @@ def forward(config, W, tokens, return_layers=False):
         after.append(x.copy())
     logits = rms_norm(x, W["final.norm"], eps) @ W["embed"].T * config.get("logit_scale", 1.0)
     return (logits, np.stack(after)) if return_layers else logits
+
+
+def greedy_generate(config, W, prompt, n):
+    """The n tokens that follow ``prompt`` when the most likely token is taken every time (the lowest id among equals)."""
+    ids = list(prompt)
+    for _ in range(n):
+        ids.append(int(np.argmax(forward(config, W, ids)[-1])))
+    return ids[len(prompt):]
