@@ -100,13 +100,14 @@ PODURAX_SIZES = {
 # mixture of experts with a gated shared expert) with the framework's closest model, the Podurax design, at equal width, depth,
 # heads, window, feed-forward work (two matrices of 1.5 x the inner size against the gated feed-forward's three) and order of
 # attention and recurrence.  ``pattern``: "a" attention, "g" the recurrence.
-def _tabatar_shape(width, layers, heads, kv_heads, dim, window, ff, g_heads, g_dim, g_vdim, rank, pattern, moe=None, streams=4, vocab=32000):
+def _tabatar_shape(width, layers, heads, kv_heads, dim, window, ff, g_heads, g_dim, g_vdim, rank, pattern, moe=None, streams=4, vocab=32000,
+                   moe_every=2):
     att = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
            "rot": {"base": 5e5, "dims": dim // 2, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 4096}}, "mask": {"size": window}}
     gla = {"heads": g_heads, "dim": g_dim, "vdim": g_vdim, "tau": 16.0, "rank": rank}
     mix = {"a": ("attention", att), "g": ("gla", gla)}
     dense = {"kind": "dense", "ff": ff}
-    mlp = lambda i: dense if moe is None or i % 2 == 0 else {"kind": "moe", "expert": {"ff": moe[2]}, "router": {"experts": moe[0], "top": moe[1]},
+    mlp = lambda i: dense if moe is None or (i + 1) % moe_every else {"kind": "moe", "expert": {"ff": moe[2]}, "router": {"experts": moe[0], "top": moe[1]},
                                                               "shared": {"ff": moe[3]}}
     return {"architecture": "Tabatar", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0}, "streams": streams,
             "logit_scale": 1.0, "logit_softcap": 30.0,
@@ -127,6 +128,46 @@ TABATAR_SIZES = {
                        _podurax_shape(2048, 8, 16, 2, 128, 2048, 5632, 4096, 16, 128, "mmam")),
     "medium-one-stream": (_tabatar_shape(2048, 8, 16, 2, 128, 2048, 8448, 16, 64, 128, 128, "ggag", streams=None),
                           _podurax_shape(2048, 8, 16, 2, 128, 2048, 5632, 4096, 16, 128, "mmam")),
+}
+# Layer sizes for the comparison of the Vavadra design (attention through a latent with a sink per head and a window;
+# differential attention within blocks; the gated delta rule; a mixture of experts with identity experts and clamped
+# activations in every layer; a looped span) with the framework's closest model, the Tabatar design on one stream, at equal
+# width, depth, heads, window, experts and order of attention and recurrence.  ``pattern``: "l" attention through a latent,
+# "a" differential attention, "d" the delta rule.
+def _vavadra_shape(width, layers, heads, kv_heads, dim, window, d_heads, d_dim, d_vdim, kv_rank, rot, moe, pattern, loop=None, vocab=32000):
+    lat = {"heads": heads, "dim": dim // 2, "rot_dim": rot, "vdim": dim, "kv_rank": kv_rank, "scale": (dim // 2 + rot) ** -0.5,
+           "rot": {"base": 10000.0, "dims": rot}, "mask": {"size": window}}
+    dif = {"heads": heads, "kv_heads": kv_heads, "dim": dim // 2, "vdim": dim, "scale": (dim // 2) ** -0.5, "diff": 0.5, "mask": {"size": window}}
+    dlt = {"heads": d_heads, "kv_heads": d_heads, "dim": d_dim, "vdim": d_vdim, "conv": 4}
+    mix = {"l": ("latent_attention", lat), "a": ("attention", dif), "d": ("delta", dlt)}
+    mlp = {"kind": "moe", "expert": {"ff": moe[2], "limit": 7.0}, "router": {"experts": moe[0] - moe[4], "identity": moe[4], "top": moe[1], "scale": 1.0},
+           "shared": {"ff": moe[3], "limit": 7.0}}
+    out = {"architecture": "Vavadra", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0}, "logit_scale": 1.0,
+           "layers": [{"type": mix[pattern[i % len(pattern)]][0], "mixer": mix[pattern[i % len(pattern)]][1], "mlp": mlp} for i in range(layers)]}
+    if loop:
+        out["loop"] = dict(zip(("start", "stop", "times"), loop))
+    return out
+
+
+def _vavadra_twin(width, layers, heads, kv_heads, dim, window, g_heads, g_dim, g_vdim, rank, moe, pattern):
+    return _tabatar_shape(width, layers, heads, kv_heads, dim, window, 0, g_heads, g_dim, g_vdim, rank, pattern, moe=moe[:4], streams=None, moe_every=1)
+
+
+VAVADRA_SIZES = {
+    # (experts + identity, top, ff, shared ff, identity)
+    "small": (_vavadra_shape(1024, 8, 8, 2, 128, 1024, 8, 64, 128, 96, 32, (16, 2, 704, 704, 2), "lald"),
+              _vavadra_twin(1024, 8, 8, 2, 128, 1024, 8, 64, 128, 64, (16, 2, 704, 704), "aaag")),
+    "medium": (_vavadra_shape(2048, 8, 16, 2, 128, 2048, 16, 64, 128, 96, 32, (32, 4, 1408, 1408, 4), "lald"),
+               _vavadra_twin(2048, 8, 16, 2, 128, 2048, 16, 64, 128, 128, (32, 4, 1408, 1408), "aaag")),
+    "medium-latent": (_vavadra_shape(2048, 8, 16, 2, 128, 2048, 16, 64, 128, 96, 32, (32, 4, 1408, 1408, 4), "l"),
+                      _vavadra_twin(2048, 8, 16, 2, 128, 2048, 16, 64, 128, 128, (32, 4, 1408, 1408), "a")),
+    "medium-differential": (_vavadra_shape(2048, 8, 16, 2, 128, 2048, 16, 64, 128, 96, 32, (32, 4, 1408, 1408, 4), "a"),
+                            _vavadra_twin(2048, 8, 16, 2, 128, 2048, 16, 64, 128, 128, (32, 4, 1408, 1408), "a")),
+    "medium-delta": (_vavadra_shape(2048, 8, 16, 2, 128, 2048, 16, 64, 128, 96, 32, (32, 4, 1408, 1408, 4), "d"),
+                     _vavadra_twin(2048, 8, 16, 2, 128, 2048, 16, 64, 128, 128, (32, 4, 1408, 1408), "g")),
+    # a latent as wide as large models of this kind have it, and the looped span (layers 2 .. 5 twice: 12 layer runs)
+    "medium-wide-latent-looped": (_vavadra_shape(2048, 8, 16, 2, 128, 2048, 16, 64, 128, 512, 64, (32, 4, 1408, 1408, 4), "lald", loop=(2, 6, 2)),
+                                  _vavadra_twin(2048, 8, 16, 2, 128, 2048, 16, 64, 128, 128, (32, 4, 1408, 1408), "aaag")),
 }
 CONTEXT = 4096
 PROMPT = 2048
@@ -151,15 +192,16 @@ def main() -> int:
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--no-gemm-tuning", action="store_true", help="leave the library's default kernel choice for large products")
-    ap.add_argument("--workload", choices=["decode", "prefill", "mumusun", "podurax", "tabatar", *WORKLOADS], default="decode",
+    ap.add_argument("--workload", choices=["decode", "prefill", "mumusun", "podurax", "tabatar", "vavadra", *WORKLOADS], default="decode",
                     help="decode: the headline measurement; prefill: only the 2,048-token prefill, --steps times "
                          "(for profiles); mixed3b / long14b: whole workloads through the scheduler; mumusun: prefill and "
                          "decode of the Mumusun design beside the dense decoder at equal size (--size, --only-design); podurax: the same "
-                         "for the Podurax design; tabatar: the Tabatar design beside the Podurax design at equal size")
-    ap.add_argument("--size", choices=["all", *dict.fromkeys([*DESIGN_SIZES, *PODURAX_SIZES, *TABATAR_SIZES])], default="all",
-                    help="--workload mumusun / podurax / tabatar: which of its sizes")
-    ap.add_argument("--only-design", choices=["both", "mumusun", "podurax", "tabatar", "dense"], default="both",
-                    help="--workload mumusun / podurax / tabatar: which of the two models")
+                         "for the Podurax design; tabatar: the Tabatar design beside the Podurax design at equal size; vavadra: the "
+                         "Vavadra design beside the Tabatar design (on one stream) at equal size")
+    ap.add_argument("--size", choices=["all", *dict.fromkeys([*DESIGN_SIZES, *PODURAX_SIZES, *TABATAR_SIZES, *VAVADRA_SIZES])], default="all",
+                    help="--workload mumusun / podurax / tabatar / vavadra: which of its sizes")
+    ap.add_argument("--only-design", choices=["both", "mumusun", "podurax", "tabatar", "vavadra", "dense"], default="both",
+                    help="--workload mumusun / podurax / tabatar / vavadra: which of the two models")
     ap.add_argument("--no-decode-weight-copy", action="store_true",
                     help="decode from the weights' plain rows instead of the tiled copy")
     ap.add_argument("--ceilings", action=argparse.BooleanOptionalAction, default=True,
@@ -200,6 +242,8 @@ def main() -> int:
         return run_design_compare(args, PODURAX_SIZES, "podurax")
     if args.workload == "tabatar":
         return run_design_compare(args, TABATAR_SIZES, "tabatar", twin="podurax")
+    if args.workload == "vavadra":
+        return run_design_compare(args, VAVADRA_SIZES, "vavadra", twin="tabatar")
     if args.workload == "mumusun":
         return run_design_compare(args)
     shape = dict({"7b": SHAPE_7B, "3b": SHAPE_3B, "14b": SHAPE_14B, "1.5b": SHAPE_15B, "0.5b": SHAPE_05B, "32b": SHAPE_32B,

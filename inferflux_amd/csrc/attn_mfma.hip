@@ -325,7 +325,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[r] = fmaf(wgt, v[r], acc[r]);
       }
-      const float inv = finish_factor(M, L, a.has_sink, a.sink_l2, a.gate, (size_t)row * a.nH + kvh * ratio + qt + c);
+      const float inv = finish_factor(M, L, a.has_sink, a.sink_l2, a.gate, (size_t)row * a.nH + kvh * ratio + qt + c, a.sinks, a.nH);
       bf16x4 w4;
 #pragma unroll
       for (int r = 0; r < 4; ++r) w4[r] = (__bf16)(acc[r] * inv);
@@ -343,7 +343,7 @@ extern "C" int ifx_attn_rows(const void* q, const void* k_cache, const void* v_c
                              const int* row_req, const int* positions, const int* block_table, int max_blocks,
                              int n_rows, int nH, int nKV, int d, int page_size, int window, int chunk,
                              int max_splits, float scale, float* part_o, float* part_ml, int waves, int req_is_row,
-                             int keep_first, int has_sink, float sink_score, const float* gate, void* stream) {
+                             int keep_first, int has_sink, float sink_score, const float* gate, const float* sinks, void* stream) {
   IFX_REQUIRE(d == D, "attn_rows: built for head_dim %d, called with %d", D, d);
   IFX_REQUIRE(n_rows >= 0 && nH > 0 && nKV > 0 && nH % nKV == 0, "attn_rows: bad head counts nH=%d nKV=%d", nH, nKV);
   IFX_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_rows: page_size %d must be a multiple of 16", page_size);
@@ -352,7 +352,7 @@ extern "C" int ifx_attn_rows(const void* q, const void* k_cache, const void* v_c
   if (n_rows == 0) return 0;
   RowArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, rows, row_req, positions, block_table,
             part_o, part_ml, (bf16_t*)out, max_blocks, n_rows, nH, nKV, page_size, window, chunk, max_splits,
-            scale * 1.4426950408889634f, 0, waves, req_is_row, window > 0 ? keep_first : 0, has_sink, sink_score * 1.4426950408889634f, gate};
+            scale * 1.4426950408889634f, 0, waves, req_is_row, window > 0 ? keep_first : 0, has_sink, sink_score * 1.4426950408889634f, gate, sinks};
   IFX_REQUIRE(keep_first >= 0, "attn_rows: keep_first %d", keep_first);
   hipStream_t s = (hipStream_t)stream;
   const bool streaming = n_rows >= ROW_STREAM_MIN_ROWS && page_size == 16;
@@ -429,6 +429,7 @@ struct TileArgs {
   int has_sink = 0;
   float sink_l2 = 0.f;
   const float* gate = nullptr;
+  const float* sinks = nullptr;
 };
 
 constexpr int N_PIECES = TK * (D / 8);                // 16-byte pieces of a K tile, and as many of a V^T tile
@@ -746,7 +747,7 @@ void attn_tiles_kernel(TileArgs a) {
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) *(floatx4*)(po + 16 * dt + 4 * g4) = q[qt].o[dt];
     } else {
-      const float inv = finish_factor(q[qt].m * a.scale_log2e, l, a.has_sink, a.sink_l2, a.gate, row * a.nH + head);
+      const float inv = finish_factor(q[qt].m * a.scale_log2e, l, a.has_sink, a.sink_l2, a.gate, row * a.nH + head, a.sinks, a.nH);
       bf16_t* orow = a.out + (row * a.nH + head) * D;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
@@ -769,7 +770,7 @@ extern "C" int ifx_attn_tiles(const void* q, const void* k_cache, const void* v_
                               int nH, int nKV, int d, int page_size, int window, float scale, int chunk, int max_splits,
                               float* part_o, float* part_ml, const int* rows, int n_rows, const int* row_req,
                               const int* positions, const int* order, int order_per_xcd, int n_xcd, int keep_first,
-                              int has_sink, float sink_score, const float* gate, void* stream) {
+                              int has_sink, float sink_score, const float* gate, const float* sinks, void* stream) {
   IFX_REQUIRE(d == D, "attn_tiles: built for head_dim %d, called with %d", D, d);
   IFX_REQUIRE(keep_first >= 0, "attn_tiles: keep_first %d", keep_first);
   IFX_REQUIRE(n_tiles >= 0 && nH > 0 && nKV > 0 && nH % nKV == 0, "attn_tiles: bad head counts nH=%d nKV=%d", nH, nKV);
@@ -786,7 +787,7 @@ extern "C" int ifx_attn_tiles(const void* q, const void* k_cache, const void* v_
   TileArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, tile_req, tile_q0, q_start,
              q_len, kv_len, block_table, max_blocks, nH, nKV, page_size, window, scale * 1.4426950408889634f, page_shift,
              n_tiles, 0, n_xcd, chunk, max_splits, part_o, part_ml, order, window > 0 ? keep_first : 0, has_sink,
-             sink_score * 1.4426950408889634f, gate};
+             sink_score * 1.4426950408889634f, gate, sinks};
   const long long items = (long long)n_tiles * nH * max_splits;
   IFX_REQUIRE(items <= (1LL << 30), "attn_tiles: too many tiles for one launch");
   IFX_REQUIRE(!order || (order_per_xcd > 0 && (long long)n_xcd * order_per_xcd >= items && order_per_xcd <= items),
@@ -799,7 +800,7 @@ extern "C" int ifx_attn_tiles(const void* q, const void* k_cache, const void* v_
   if (max_splits > 1) {
     RowArgs m{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, rows, row_req, positions, block_table,
               part_o, part_ml, (bf16_t*)out, max_blocks, n_rows, nH, nKV, page_size, window, chunk, max_splits,
-              scale * 1.4426950408889634f, 1, 0, 0, window > 0 ? keep_first : 0, has_sink, sink_score * 1.4426950408889634f, gate};
+              scale * 1.4426950408889634f, 1, 0, 0, window > 0 ? keep_first : 0, has_sink, sink_score * 1.4426950408889634f, gate, sinks};
     hipLaunchKernelGGL(attn_rows_merge_kernel, dim3(n_rows, nH), dim3(WAVE * merge_waves(max_splits)), 0, s, m);
   }
   IFX_LAUNCH_CHECK();

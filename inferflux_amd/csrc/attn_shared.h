@@ -84,17 +84,24 @@ struct RowArgs {
   int req_is_row;         // row_req[r] == r for every row (a step of single tokens): table lookups need not wait for it
   // Optional, off when zero.  keep_first: a windowed row also sees its request's first so many keys.  has_sink: a key
   // without value whose score (times log2 e: sink_l2) joins the softmax's denominator.  gate [T, nH]: a factor on
-  // every head's output.
+  // every head's output.  sinks [nH]: a sink score for every head (as given, not yet times log2 e), instead of the one.
   int keep_first = 0;
   int has_sink = 0;
   float sink_l2 = 0.f;
   const float* gate = nullptr;
+  const float* sinks = nullptr;
 };
 
 // The sink joins a finished (maximum M, sum L, unnormalised output) once, where the output is written: returns the
 // factor on the output, 1 / (L + 2^(sink - M)) (times the head's gate), with care for a maximum below the sink's score.
-__device__ __forceinline__ float finish_factor(float M, float L, int has_sink, float sink_l2, const float* gate, size_t gate_at) {
+// ``at`` is row * nH + head; with ``sinks`` the head's own score is taken.
+__device__ __forceinline__ float finish_factor(float M, float L, int has_sink, float sink_l2, const float* gate, size_t gate_at,
+                                               const float* sinks = nullptr, int nH = 1) {
   float f = 1.f;
+  if (sinks) {
+    has_sink = 1;
+    sink_l2 = sinks[gate_at % (size_t)nH] * 1.4426950408889634f;
+  }
   if (has_sink) {
     const float Ms = fmaxf(M, sink_l2);
     f = M == -INFINITY ? 0.f : exp2f(M - Ms);
@@ -229,7 +236,7 @@ __global__ __launch_bounds__(WAVE * MERGE_MAX_WAVES) void attn_rows_merge_kernel
     }
   }
   else M_all = M;
-  const float inv = finish_factor(M_all, L, a.has_sink, a.sink_l2, a.gate, (size_t)row * a.nH + head);
+  const float inv = finish_factor(M_all, L, a.has_sink, a.sink_l2, a.gate, (size_t)row * a.nH + head, a.sinks, a.nH);
 #pragma unroll
   for (int c = 0; c < C; ++c) {
     const int e = lane + c * WAVE;

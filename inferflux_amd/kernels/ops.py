@@ -1548,12 +1548,14 @@ def _attn_common(q, k_cache, v_cache, qt=1, direct=True):
     return T, nH, d, nKV, page_size, load_module(name, variant)
 
 
-def _attn_extras(T, nH, keep_first, sink, gate):
-    """The four optional arguments of the matrix-core attention kernels: kept first keys, whether there is a sink, its
-    score, the gate's pointer."""
+def _attn_extras(T, nH, keep_first, sink, gate, sinks=None):
+    """The five optional arguments of the matrix-core attention kernels: kept first keys, whether there is a sink, its
+    score, the gate's pointer, the pointer to a sink score per head."""
     if gate is not None:
         _check(gate, "gate", (T, nH), torch.float32)
-    return int(keep_first or 0), 0 if sink is None else 1, float(sink or 0.0), _ptr(gate)
+    if sinks is not None:
+        _check(sinks, "sinks", (nH,), torch.float32)
+    return int(keep_first or 0), 0 if sink is None else 1, float(sink or 0.0), _ptr(gate), _ptr(sinks)
 
 
 ROW_MAX_WAVES = 8
@@ -1571,7 +1573,7 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
                    rows: Optional[torch.Tensor], n_rows: int, row_req: torch.Tensor, positions: torch.Tensor,
                    block_table: torch.Tensor, window: Optional[int], scale: float, chunk: int, max_splits: int,
                    waves: int = 0, req_is_row: bool = False, keep_first: int = 0, sink: Optional[float] = None,
-                   gate: Optional[torch.Tensor] = None) -> None:
+                   gate: Optional[torch.Tensor] = None, sinks: Optional[torch.Tensor] = None) -> None:
     """Attention of single rows (``rows`` int32, or None for rows 0..n_rows-1) into ``out`` [T, nH*d].  ``keep_first``,
     ``sink``, ``gate``: as for ``attention_plain``.
 
@@ -1599,11 +1601,11 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         part_ml = torch.empty((n_rows, nH, max_splits, 2), dtype=torch.float32, device=q.device)
     if req_is_row and block_table.shape[0] < T:
         raise KernelError("attention_rows: req_is_row needs a block-table row for every row of the step")
-    _call(mod, "ifx_attn_rows", (P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, P, P, I, I, I, I, F, P, P),
+    _call(mod, "ifx_attn_rows", (P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, P, P, I, I, I, I, F, P, P, P),
           q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _ptr(rows), row_req.data_ptr(),
           positions.data_ptr(), block_table.data_ptr(), block_table.shape[1], n_rows, nH, nKV, d, page_size,
           int(window or 0), chunk, max_splits, float(scale), _ptr(part_o), _ptr(part_ml), waves, 1 if req_is_row else 0,
-          *_attn_extras(T, nH, keep_first, sink, gate), _stream())
+          *_attn_extras(T, nH, keep_first, sink, gate, sinks), _stream())
 
 
 def attention_tile_rows(head_dim: int, qt: int = 1) -> int:
@@ -1618,7 +1620,7 @@ def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                     qt: int = 1, chunk: int = 0, max_splits: int = 1, rows: Optional[torch.Tensor] = None,
                     row_req: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None,
                     order: Optional[torch.Tensor] = None, keep_first: int = 0, sink: Optional[float] = None,
-                    gate: Optional[torch.Tensor] = None) -> None:
+                    gate: Optional[torch.Tensor] = None, sinks: Optional[torch.Tensor] = None) -> None:
     """Attention of tiles of ``attention_tile_rows(d, qt)`` consecutive rows of one request each (tile t:
     request tile_req[t], rows from tile_q0[t] of that request's rows in this step) into ``out`` [T, nH*d].
 
@@ -1629,7 +1631,7 @@ def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 
     ``order`` (int32 [8 * n], from ``attention.tile_order``) says which work item each workgroup of the launch
     takes; every item must appear exactly once (-1: a workgroup without work).  The result does not depend on it."""
-    extras = bool(keep_first) or sink is not None or gate is not None      # (the kernel that loads straight into LDS has none of them)
+    extras = bool(keep_first) or sink is not None or gate is not None or sinks is not None      # (the kernel that loads straight into LDS has none of them)
     T, nH, d, nKV, page_size, mod = _attn_common(q, k_cache, v_cache, qt, not extras)
     _, _, entry, rows_fn = _tile_module(d, qt, not extras)
     if mod.fn(rows_fn, ())() != attention_tile_rows(d, qt):
@@ -1667,7 +1669,7 @@ def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             _ptr(part_o), _ptr(part_ml), _ptr(rows), n_rows, _ptr(row_req), _ptr(positions), _ptr(order), per_xcd, N_XCD)
     types = (P, P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, F, I, I, P, P, P, I, P, P, P, I, I)
     if entry == "ifx_attn_tiles":
-        _call(mod, entry, types + (I, I, F, P, P), *args, *_attn_extras(T, nH, keep_first, sink, gate), _stream())
+        _call(mod, entry, types + (I, I, F, P, P, P), *args, *_attn_extras(T, nH, keep_first, sink, gate, sinks), _stream())
     else:
         _call(mod, entry, types + (P,), *args, _stream())
 

@@ -71,7 +71,7 @@ class LatentAttention(Mixer):
         side too, rot_dim / (kv_rank + rot_dim) more bytes and products on that side, and what comes back behind a
         head's kv_rank sums is left unread."""
         d = self.kv_rank + self.rot_dim
-        return d if (d % 16 == 0 and d <= ops.MFMA_MAX_HEAD_DIM and not self.sinks) else self.kv_rank
+        return d if (d % 16 == 0 and d <= ops.MFMA_MAX_HEAD_DIM) else self.kv_rank
 
     def cache_spec(self) -> CacheSpec:
         d, dv = self.kv_rank + self.rot_dim, self.value_width
