@@ -140,12 +140,12 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
   // A step in which every request brings one row (a decode step) says so: the row's request is the row itself, and
   // without a window a split's first key does not depend on the row's position, so the split's block-table entries
   // are asked for together with the position instead of after it (one trip to memory fewer before the first keys).
-  const bool early = a.req_is_row && a.window <= 0;
+  const bool early = a.req_is_row && a.window <= 0 && a.block <= 0;
   const int* early_table = a.block_table + (size_t)row * a.max_blocks;
   const int early_base = split * a.chunk / a.P;
   const int early_pages = (early && early_base + lane < a.max_blocks) ? early_table[early_base + lane] : -1;
   const int pos = a.positions[row];
-  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int lo = first_seen(pos, a.window, a.block);
   const int ka = max(lo, split * a.chunk), kb = min(pos + 1, (split + 1) * a.chunk);  // keys [ka, kb)
   // ... and of the kept first keys [0, keep) those of this split: [split * chunk, ke).  Where there are any the walk
   // starts at the split's first key and passes whatever lies between them and the window without loading it.
@@ -236,7 +236,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int W = a.waves, n_threads = W * WAVE;
   const int row = a.rows ? a.rows[ri] : ri;
   const int pos = a.positions[row];
-  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int lo = first_seen(pos, a.window, a.block);
   // this wave's keys: the visible ones from the first visible run of 32 on, in W equal shares of whole runs.  With
   // kept first keys [0, keep) before the window the runs are numbered as if the window's first run followed the last
   // kept run: walk place v is key v below kr and key v + gap from there on.
@@ -343,7 +343,7 @@ extern "C" int ifx_attn_rows(const void* q, const void* k_cache, const void* v_c
                              const int* row_req, const int* positions, const int* block_table, int max_blocks,
                              int n_rows, int nH, int nKV, int d, int page_size, int window, int chunk,
                              int max_splits, float scale, float* part_o, float* part_ml, int waves, int req_is_row,
-                             int keep_first, int has_sink, float sink_score, const float* gate, const float* sinks, void* stream) {
+                             int keep_first, int has_sink, float sink_score, const float* gate, const float* sinks, int block, void* stream) {
   IFX_REQUIRE(d == D, "attn_rows: built for head_dim %d, called with %d", D, d);
   IFX_REQUIRE(n_rows >= 0 && nH > 0 && nKV > 0 && nH % nKV == 0, "attn_rows: bad head counts nH=%d nKV=%d", nH, nKV);
   IFX_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_rows: page_size %d must be a multiple of 16", page_size);
@@ -352,7 +352,7 @@ extern "C" int ifx_attn_rows(const void* q, const void* k_cache, const void* v_c
   if (n_rows == 0) return 0;
   RowArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, rows, row_req, positions, block_table,
             part_o, part_ml, (bf16_t*)out, max_blocks, n_rows, nH, nKV, page_size, window, chunk, max_splits,
-            scale * 1.4426950408889634f, 0, waves, req_is_row, window > 0 ? keep_first : 0, has_sink, sink_score * 1.4426950408889634f, gate, sinks};
+            scale * 1.4426950408889634f, 0, waves, req_is_row, window > 0 ? keep_first : 0, has_sink, sink_score * 1.4426950408889634f, gate, sinks, block};
   IFX_REQUIRE(keep_first >= 0, "attn_rows: keep_first %d", keep_first);
   hipStream_t s = (hipStream_t)stream;
   const bool streaming = n_rows >= ROW_STREAM_MIN_ROWS && page_size == 16;
@@ -430,6 +430,7 @@ struct TileArgs {
   float sink_l2 = 0.f;
   const float* gate = nullptr;
   const float* sinks = nullptr;
+  int block = 0;          // > 0: a row sees only the keys of its own block of so many positions (see first_seen)
 };
 
 constexpr int N_PIECES = TK * (D / 8);                // 16-byte pieces of a K tile, and as many of a V^T tile
@@ -674,7 +675,7 @@ void attn_tiles_kernel(TileArgs a) {
   const int rows_here = min(TQ, qlen - q0);
   const int pos_first = start + q0, row_last = pos_first + rows_here - 1;
   // the keys of this workgroup: what its rows can see, cut to its split
-  const int lo_wg = max(a.window > 0 ? max(0, pos_first - a.window + 1) : 0, a.max_splits > 1 ? split * a.chunk : 0);
+  const int lo_wg = max(first_seen(pos_first, a.window, a.block), a.max_splits > 1 ? split * a.chunk : 0);
   const int pos_last = a.max_splits > 1 ? min(row_last, (split + 1) * a.chunk - 1) : row_last;
 
   // this wave's rows: QT tiles of 16, lane `col` of tile qt holds row 16 * QT * wid + 16 * qt + col of the tile
@@ -686,7 +687,7 @@ void attn_tiles_kernel(TileArgs a) {
     const int my_q = wave_q + 16 * qt + col;
     q[qt].ok = my_q < qlen;
     q[qt].pos = start + my_q;
-    q[qt].lo = a.window > 0 ? max(0, q[qt].pos - a.window + 1) : 0;
+    q[qt].lo = first_seen(q[qt].pos, a.window, a.block);
     q[qt].m = -INFINITY;
     q[qt].l = 0.f;
 #pragma unroll
@@ -700,7 +701,7 @@ void attn_tiles_kernel(TileArgs a) {
   // the keys this wave's rows can see at all: tiles outside are skipped by the whole wave
   const int wave_first = start + wave_q;
   const int wave_hi = min(row_last, wave_first + 16 * QT - 1);
-  const int wave_lo = a.window > 0 ? max(0, wave_first - a.window + 1) : 0;
+  const int wave_lo = first_seen(wave_first, a.window, a.block);
 
   // The walk: key tiles from the window's first to the last row's, and before them, where the rows keep their
   // request's first keys [0, keep) and those end before the window's first tile, the tiles that hold them (of this
@@ -731,7 +732,7 @@ void attn_tiles_kernel(TileArgs a) {
     if (j0 > wave_hi || (j0 + TK <= wave_lo && j0 >= keep)) continue;   // uniform over the wave; barriers are at the loop's top
 
     // A tile every key of which every row of this wave sees needs no mask: the common case.
-    const bool full = j0 + TK - 1 <= wave_first && (a.window <= 0 || j0 >= wave_hi - a.window + 1);
+    const bool full = j0 + TK - 1 <= wave_first && j0 >= first_seen(wave_hi, a.window, a.block);
     if (full) tile_math<false>(k_s, v_s, q, a.scale_log2e, j0, col, g4);
     else tile_math<true>(k_s, v_s, q, a.scale_log2e, j0, col, g4, keep);
   }
@@ -770,7 +771,7 @@ extern "C" int ifx_attn_tiles(const void* q, const void* k_cache, const void* v_
                               int nH, int nKV, int d, int page_size, int window, float scale, int chunk, int max_splits,
                               float* part_o, float* part_ml, const int* rows, int n_rows, const int* row_req,
                               const int* positions, const int* order, int order_per_xcd, int n_xcd, int keep_first,
-                              int has_sink, float sink_score, const float* gate, const float* sinks, void* stream) {
+                              int has_sink, float sink_score, const float* gate, const float* sinks, int block, void* stream) {
   IFX_REQUIRE(d == D, "attn_tiles: built for head_dim %d, called with %d", D, d);
   IFX_REQUIRE(keep_first >= 0, "attn_tiles: keep_first %d", keep_first);
   IFX_REQUIRE(n_tiles >= 0 && nH > 0 && nKV > 0 && nH % nKV == 0, "attn_tiles: bad head counts nH=%d nKV=%d", nH, nKV);
@@ -787,7 +788,7 @@ extern "C" int ifx_attn_tiles(const void* q, const void* k_cache, const void* v_
   TileArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, tile_req, tile_q0, q_start,
              q_len, kv_len, block_table, max_blocks, nH, nKV, page_size, window, scale * 1.4426950408889634f, page_shift,
              n_tiles, 0, n_xcd, chunk, max_splits, part_o, part_ml, order, window > 0 ? keep_first : 0, has_sink,
-             sink_score * 1.4426950408889634f, gate, sinks};
+             sink_score * 1.4426950408889634f, gate, sinks, block};
   const long long items = (long long)n_tiles * nH * max_splits;
   IFX_REQUIRE(items <= (1LL << 30), "attn_tiles: too many tiles for one launch");
   IFX_REQUIRE(!order || (order_per_xcd > 0 && (long long)n_xcd * order_per_xcd >= items && order_per_xcd <= items),
@@ -800,7 +801,7 @@ extern "C" int ifx_attn_tiles(const void* q, const void* k_cache, const void* v_
   if (max_splits > 1) {
     RowArgs m{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, rows, row_req, positions, block_table,
               part_o, part_ml, (bf16_t*)out, max_blocks, n_rows, nH, nKV, page_size, window, chunk, max_splits,
-              scale * 1.4426950408889634f, 1, 0, 0, window > 0 ? keep_first : 0, has_sink, sink_score * 1.4426950408889634f, gate, sinks};
+              scale * 1.4426950408889634f, 1, 0, 0, window > 0 ? keep_first : 0, has_sink, sink_score * 1.4426950408889634f, gate, sinks, block};
     hipLaunchKernelGGL(attn_rows_merge_kernel, dim3(n_rows, nH), dim3(WAVE * merge_waves(max_splits)), 0, s, m);
   }
   IFX_LAUNCH_CHECK();

@@ -90,7 +90,14 @@ struct RowArgs {
   float sink_l2 = 0.f;
   const float* gate = nullptr;
   const float* sinks = nullptr;
+  int block = 0;          // > 0: a row sees only the keys of its own block of so many positions, counted from position 0
 };
+
+// The first position a row at ``pos`` sees: the start of its window, and of its block where the sequence is cut into blocks.
+__device__ __forceinline__ int first_seen(int pos, int window, int block) {
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  return block > 0 ? max(lo, pos - pos % block) : lo;
+}
 
 // The sink joins a finished (maximum M, sum L, unnormalised output) once, where the output is written: returns the
 // factor on the output, 1 / (L + 2^(sink - M)) (times the head's gate), with care for a maximum below the sink's score.
@@ -134,7 +141,7 @@ __global__ __launch_bounds__(WAVE * MERGE_MAX_WAVES) void attn_rows_merge_kernel
   const int ri = blockIdx.x, head = blockIdx.y, lane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE, nw = blockDim.x / WAVE;
   const int row = a.rows ? a.rows[ri] : ri;
   const int pos = a.positions[row];
-  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int lo = first_seen(pos, a.window, a.block);
   // first and last split that hold a visible key (with kept first keys the walk starts at split 0: the splits between
   // them and the window saw nothing and say so)
   const int first = (a.keep_first > 0 && lo > 0) ? 0 : lo / a.chunk, last = pos / a.chunk;

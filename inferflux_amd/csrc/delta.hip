@@ -13,19 +13,20 @@
 // its logarithms, S, every sum, the norm and the gate are float whatever that type is.
 //
 // A request's S lives in its state slot, float32, at ``state_offset`` floats into the slot's row, laid out
-// [head][value column][d_pad] with d_pad = CH * KS >= d.  A workgroup is one head of one request; thread (column j, run
-// s) holds CH consecutive key channels of column j in registers, the KS threads of a column are neighbouring lanes and
-// add their parts of S^T k and S^T q by butterfly shuffles (a fixed order).  Tokens are taken STAGE at a time: all
-// threads load the stage's q, k, v into LDS, a wave per (token, vector) forms the unit norms, a thread per token beta
-// and the decay; everybody walks the stage's tokens; a wave per token norms and gates o.  The order of a token's
-// operations does not depend on how the request was cut into steps, so results are bit-equal across cuttings.
+// [head][value column][d_pad] with d_pad = CH * KS >= d.  The columns of S never meet (column j is only ever read and
+// written with v_j, u_j and o_j), so a head's columns are dealt to several workgroups of ``cols`` columns each, which
+// spreads one request over many compute units.  In a workgroup thread (column j, run s) holds CH consecutive key channels
+// of column j in registers; the KS threads of a column are neighbouring lanes and add their parts of S^T k and S^T q by
+// butterfly shuffles (a fixed order).  Tokens are taken STAGE at a time: all threads load the stage's q, k and their
+// columns of v into LDS (the next stage's are asked for before the walk and land in registers meanwhile), a few lanes per
+// (token, vector) form the unit norms, a thread per token beta and the decay; everybody walks the stage's tokens and
+// leaves o in LDS, from where it goes to ``o_raw`` [T, H dv] (float).  A second kernel, a wave per (token, head), norms and
+// gates o.  The order of a token's operations does not depend on how the request was cut into steps, so results are
+// bit-equal across cuttings.
 #include "common.h"
 
 IFX_DEFINE_LAST_ERROR()
 
-#define STAGE 8
-#define MAX_DPAD 256
-#define MAX_DV 512
 
 struct DeltaArgs {
   const void* u;          // [T, ldu]: q (G d) | k (G d) | v (H dv)
@@ -41,97 +42,171 @@ struct DeltaArgs {
   size_t state_stride, state_offset;
   const int* q_start; const int* q_len; const int* slots;     // [R]
   void* out;              // [T, H dv]
-  int H, G, d, dv, KS;
+  float* o_raw;           // [T, H dv]: the read-outs before their norm and gate
+  int T, H, G, d, dv, KS, cols;
 };
 
 __device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 
+#define STAGE 16
+#define MAX_DPAD 256
+#define MAX_COLS 128
+#define MAX_PRE 16          // 16-byte-free prefetch: values a thread holds for the next stage (see below)
+
+// The sum over the KS (a power of two) neighbouring lanes that share a column, in every one of them: neighbours within a
+// row of 16 lanes swap through the lanes' own data paths (pairs, quads, mirrored halves of 8, mirrored rows of 16: a few
+// cycles each, where a trip through the LDS crossbar costs a token's whole arithmetic); wider groups go on by shuffles.
+// The order of the additions is fixed by the lane numbers.
+#define DPP_ADD(v, ctrl) (v) += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), (ctrl), 0xF, 0xF, true))
+__device__ __forceinline__ float column_sum(float v, int KS) {
+  if (KS >= 2) DPP_ADD(v, 0xB1);        // quad_perm [1, 0, 3, 2]
+  if (KS >= 4) DPP_ADD(v, 0x4E);        // quad_perm [2, 3, 0, 1]
+  if (KS >= 8) DPP_ADD(v, 0x141);       // row_half_mirror
+  if (KS >= 16) DPP_ADD(v, 0x140);      // row_mirror
+  if (KS >= 32) v += __shfl_xor(v, 16, WAVE);
+  if (KS >= 64) v += __shfl_xor(v, 32, WAVE);
+  return v;
+}
+
+// A workgroup's meeting point for what it wrote to LDS: waits for the wave's own LDS operations and for the others, but
+// not for loads from memory that are still on their way into registers (the next stage's), as __syncthreads() would.
+#define LDS_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
+
 template <typename T, int CH>
-__global__ __launch_bounds__(1024) void delta_kernel(DeltaArgs a) {
+__global__ __launch_bounds__(256) void delta_kernel(DeltaArgs a) {
   __shared__ float q_s[STAGE][MAX_DPAD], k_s[STAGE][MAX_DPAD];
-  __shared__ float v_s[STAGE][MAX_DV], o_s[STAGE][MAX_DV];
+  __shared__ float v_s[STAGE][MAX_COLS], o_s[STAGE][MAX_COLS];
   __shared__ float beta_s[STAGE], g_s[STAGE];
-  const int h = blockIdx.x, r = blockIdx.y;
+  const int n_cb = (a.dv + a.cols - 1) / a.cols;
+  const int h = blockIdx.x / n_cb, j0 = (blockIdx.x % n_cb) * a.cols, r = blockIdx.y;
   const int n = a.q_len[r];
   if (n <= 0) return;
   const int t0 = a.q_start[r];
   const int d = a.d, dv = a.dv, KS = a.KS, dpad = CH * KS;
+  const int cols = min(a.cols, dv - j0);
   const int g = h / (a.H / a.G);
   const int tid = threadIdx.x, nthr = blockDim.x;
   const int wid = tid / WAVE, lane = tid % WAVE, nw = (nthr + WAVE - 1) / WAVE;
-  const int j = tid / KS, s = tid % KS;              // this thread's column of S and its run of channels
-  const bool owner = j < dv;
-  float* Sp = a.state + (size_t)a.slots[r] * a.state_stride + a.state_offset + ((size_t)h * dv + (owner ? j : 0)) * dpad + s * CH;
+  const int jl = tid / KS, s = tid % KS;             // this thread's column (within the workgroup's) and its run of channels
+  const bool owner = jl < cols;
+  float* Sp = a.state + (size_t)a.slots[r] * a.state_stride + a.state_offset + ((size_t)h * dv + j0 + (owner ? jl : 0)) * dpad + s * CH;
   float S[CH];
 #pragma unroll
   for (int i = 0; i < CH; ++i) S[i] = owner ? Sp[i] : 0.f;
   const T* u = (const T*)a.u;
   const T* rows = (const T*)a.rows;
   const float decay_rate = expf(a.A_log[h]), dt_b = a.dt_bias[h], q_mult = 1.0f / sqrtf((float)d);
-
-  for (int base = 0; base < n; base += STAGE) {
+  const int NL = nthr >= 256 ? 8 : (nthr >= 128 ? 4 : 2);      // lanes to a (token, vector) pair of a stage's 2 STAGE unit norms
+  // What a thread fetches of a stage: elements x = tid, tid + nthr, ... of the stage's (token, channel) pairs of q and of k
+  // and of its (token, column) pairs of v.  STAGE * dpad and STAGE * cols are at most MAX_PRE * nthr.
+  // (dpad is a power of two; the places of a thread's v elements are the same in every stage and found once)
+  const int per_qk = (STAGE * dpad + nthr - 1) / nthr, per_v = (STAGE * cols + nthr - 1) / nthr;
+  const int dshift = __ffs(dpad) - 1;
+  int v_tt[MAX_PRE], v_c[MAX_PRE];
+#pragma unroll
+  for (int e = 0; e < MAX_PRE; ++e) {
+    const int x = tid + e * nthr;
+    v_tt[e] = e < per_v ? x / cols : STAGE;
+    v_c[e] = e < per_v ? x % cols : 0;
+  }
+  float pq[MAX_PRE], pk[MAX_PRE], pv[MAX_PRE], pb = 0.f, pg = 0.f;
+  auto fetch = [&](int base) {
     const int cnt = min(STAGE, n - base);
-    __syncthreads();            // the last stage's output pass is done with o_s, its walk with q_s, k_s, v_s
-    for (int x = tid; x < cnt * dpad; x += nthr) {
-      const int tt = x / dpad, c = x % dpad;
-      const size_t row = (size_t)(t0 + base + tt) * a.ldu;
-      q_s[tt][c] = c < d ? to_f(u[row + (size_t)g * d + c]) : 0.f;
-      k_s[tt][c] = c < d ? to_f(u[row + (size_t)(a.G + g) * d + c]) : 0.f;
+#pragma unroll
+    for (int e = 0; e < MAX_PRE; ++e) {
+      if (e >= per_qk) break;
+      const int x = tid + e * nthr, tt = x >> dshift, c = x & (dpad - 1);
+      const bool in = tt < cnt && c < d;
+      const size_t row = (size_t)(t0 + base + (in ? tt : 0)) * a.ldu;
+      pq[e] = in ? to_f(u[row + (size_t)g * d + c]) : 0.f;
+      pk[e] = in ? to_f(u[row + (size_t)(a.G + g) * d + c]) : 0.f;
     }
-    for (int x = tid; x < cnt * dv; x += nthr) {
-      const int tt = x / dv, c = x % dv;
-      v_s[tt][c] = to_f(u[(size_t)(t0 + base + tt) * a.ldu + (size_t)2 * a.G * d + (size_t)h * dv + c]);
+#pragma unroll
+    for (int e = 0; e < MAX_PRE; ++e) {
+      if (e >= per_v) break;
+      const int tt = v_tt[e], c = v_c[e];
+      const bool in = tt < cnt;
+      pv[e] = in ? to_f(u[(size_t)(t0 + base + tt) * a.ldu + (size_t)2 * a.G * d + (size_t)h * dv + j0 + c]) : 0.f;
     }
     if (tid < cnt) {
       const size_t row = (size_t)(t0 + base + tid) * a.ldr;
-      beta_s[tid] = 1.0f / (1.0f + expf(-to_f(rows[row + a.col_b + h])));
-      g_s[tid] = expf(-decay_rate * softplus_f(to_f(rows[row + a.col_a + h]) + dt_b));
+      pb = to_f(rows[row + a.col_b + h]);
+      pg = to_f(rows[row + a.col_a + h]);
     }
-    __syncthreads();
-    // unit norms: a wave per (token, q or k); the lanes' squares added by the wave's butterfly
-    for (int x = wid; x < 2 * cnt; x += nw) {
-      float* vec = (x & 1) ? k_s[x >> 1] : q_s[x >> 1];
+  };
+  fetch(0);
+  for (int base = 0; base < n; base += STAGE) {
+    const int cnt = min(STAGE, n - base);
+    LDS_BARRIER();              // the last stage's walk is done with q_s, k_s, v_s, its write-out with o_s
+#pragma unroll
+    for (int e = 0; e < MAX_PRE; ++e) {
+      if (e >= per_qk) break;
+      const int x = tid + e * nthr;
+      if (x < STAGE * dpad) { q_s[x >> dshift][x & (dpad - 1)] = pq[e]; k_s[x >> dshift][x & (dpad - 1)] = pk[e]; }
+    }
+#pragma unroll
+    for (int e = 0; e < MAX_PRE; ++e) {
+      if (e >= per_v) break;
+      if (v_tt[e] < STAGE) v_s[v_tt[e]][v_c[e]] = pv[e];
+    }
+    if (tid < cnt) {
+      beta_s[tid] = 1.0f / (1.0f + expf(-pb));
+      g_s[tid] = expf(-decay_rate * softplus_f(pg + dt_b));
+    }
+    LDS_BARRIER();
+    if (base + STAGE < n) fetch(base + STAGE);          // the next stage's loads are on their way during the norms and the walk
+    // unit norms: NL neighbouring lanes per (token, q or k), all pairs at once; the lanes' squares added by column_sum
+    {
+      const int pair = tid / NL, l = tid % NL;
+      float* vec = (pair & 1) ? k_s[min(pair >> 1, STAGE - 1)] : q_s[min(pair >> 1, STAGE - 1)];
+      const bool mine = pair < 2 * cnt;
       float ss = 0.f;
-      for (int c = lane; c < d; c += WAVE) ss = fmaf(vec[c], vec[c], ss);
-      const float f = ((x & 1) ? 1.0f : q_mult) / sqrtf(wave_sum(ss) + 1e-6f);
-      for (int c = lane; c < d; c += WAVE) vec[c] *= f;
+      if (mine)
+        for (int c = l; c < d; c += NL) ss = fmaf(vec[c], vec[c], ss);
+      ss = column_sum(ss, NL);
+      if (mine) {
+        const float f = ((pair & 1) ? 1.0f : q_mult) / sqrtf(ss + 1e-6f);
+        for (int c = l; c < d; c += NL) vec[c] *= f;
+      }
     }
-    __syncthreads();
+    LDS_BARRIER();
     if (owner) {
+      // a token's k, q, v, decay and beta are read from LDS while the token before it is worked on; the sums over a
+      // thread's channels run in four chains that are added at the end (a fixed order)
+      float kn[CH], qn[CH], vn = v_s[0][jl], gn = g_s[0], bn = beta_s[0];
+#pragma unroll
+      for (int i = 0; i < CH; ++i) { kn[i] = k_s[0][s * CH + i]; qn[i] = q_s[0][s * CH + i]; }
       for (int tt = 0; tt < cnt; ++tt) {
-        const float gd = g_s[tt], bt = beta_s[tt];
-        const float* kk = k_s[tt] + s * CH;
-        const float* qq = q_s[tt] + s * CH;
-        float pred = 0.f;
+        float kk[CH], qq[CH];
+        const float gd = gn, bt = bn, vt = vn;
+#pragma unroll
+        for (int i = 0; i < CH; ++i) { kk[i] = kn[i]; qq[i] = qn[i]; }
+        if (tt + 1 < cnt) {
+          vn = v_s[tt + 1][jl]; gn = g_s[tt + 1]; bn = beta_s[tt + 1];
+#pragma unroll
+          for (int i = 0; i < CH; ++i) { kn[i] = k_s[tt + 1][s * CH + i]; qn[i] = q_s[tt + 1][s * CH + i]; }
+        }
+        float p4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < CH; ++i) {
           S[i] *= gd;
-          pred = fmaf(S[i], kk[i], pred);
+          p4[i & 3] = fmaf(S[i], kk[i], p4[i & 3]);
         }
-        for (int o = 1; o < KS; o <<= 1) pred += __shfl_xor(pred, o, WAVE);
-        const float upd = bt * (v_s[tt][j] - pred);
-        float out = 0.f;
+        const float pred = column_sum((p4[0] + p4[1]) + (p4[2] + p4[3]), KS);
+        const float upd = bt * (vt - pred);
+        float o4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < CH; ++i) {
           S[i] = fmaf(kk[i], upd, S[i]);
-          out = fmaf(S[i], qq[i], out);
+          o4[i & 3] = fmaf(S[i], qq[i], o4[i & 3]);
         }
-        for (int o = 1; o < KS; o <<= 1) out += __shfl_xor(out, o, WAVE);
-        if (s == 0) o_s[tt][j] = out;
+        const float out = column_sum((o4[0] + o4[1]) + (o4[2] + o4[3]), KS);
+        if (s == 0) o_s[tt][jl] = out;
       }
     }
-    __syncthreads();
-    // the head's norm and gate: a wave per token
-    for (int tt = wid; tt < cnt; tt += nw) {
-      float ss = 0.f;
-      for (int c = lane; c < dv; c += WAVE) ss = fmaf(o_s[tt][c], o_s[tt][c], ss);
-      const float f = 1.0f / sqrtf(wave_sum(ss) / (float)dv + a.eps);
-      const size_t row = (size_t)(t0 + base + tt);
-      for (int c = lane; c < dv; c += WAVE) {
-        const float gt = to_f(rows[row * a.ldr + a.col_g + (size_t)h * dv + c]);
-        ((T*)a.out)[(row * a.H + h) * dv + c] = from_f<T>(o_s[tt][c] * f * load_dyn(a.norm_w, a.norm_dtype, c) * act_silu(gt));
-      }
-    }
+    LDS_BARRIER();
+    for (int x = tid; x < cnt * cols; x += nthr)
+      a.o_raw[((size_t)(t0 + base + x / cols) * a.H + h) * dv + j0 + x % cols] = o_s[x / cols][x % cols];
   }
   if (owner) {
 #pragma unroll
@@ -139,22 +214,44 @@ __global__ __launch_bounds__(1024) void delta_kernel(DeltaArgs a) {
   }
 }
 
+// out[t, h, :] = o_raw[t, h, :] / sqrt(mean(o_raw[t, h, :]^2) + eps) * w * silu(gate[t, h, :]): a wave per (token, head)
+template <typename T>
+__global__ __launch_bounds__(256) void delta_finish_kernel(DeltaArgs a) {
+  const size_t item = (size_t)blockIdx.x * (256 / WAVE) + threadIdx.x / WAVE;
+  const int lane = threadIdx.x % WAVE;
+  if (item >= (size_t)a.T * a.H) return;
+  const size_t t = item / a.H;
+  const int h = (int)(item % a.H), dv = a.dv;
+  const float* o = a.o_raw + item * dv;
+  float ss = 0.f;
+  for (int c = lane; c < dv; c += WAVE) ss = fmaf(o[c], o[c], ss);
+  const float f = 1.0f / sqrtf(wave_sum(ss) / (float)dv + a.eps);
+  const T* rows = (const T*)a.rows;
+  for (int c = lane; c < dv; c += WAVE) {
+    const float gt = to_f(rows[t * a.ldr + a.col_g + (size_t)h * dv + c]);
+    ((T*)a.out)[item * dv + c] = from_f<T>(o[c] * f * load_dyn(a.norm_w, a.norm_dtype, c) * act_silu(gt));
+  }
+}
+
 extern "C" int ifx_delta_rule(const void* u, int ldu, const void* rows, int ldr, int col_g, int col_b, int col_a, int dtype,
                               const float* A_log, const float* dt_bias, const void* norm_w, int norm_dtype, float eps, float* state,
                               long long state_stride, long long state_offset, const int* q_start, const int* q_len, const int* slots,
-                              void* out, int R, int H, int G, int d, int dv, int ch, int ks, void* stream) {
+                              void* out, float* o_raw, int T, int R, int H, int G, int d, int dv, int ch, int ks, int cols, void* stream) {
   IFX_REQUIRE(R >= 0 && H > 0 && G > 0 && H % G == 0 && d > 0 && dv > 0, "delta_rule: bad sizes R=%d H=%d G=%d d=%d dv=%d", R, H, G, d, dv);
   IFX_REQUIRE(ks > 0 && ks <= WAVE && (ks & (ks - 1)) == 0, "delta_rule: %d threads to a column (a power of two up to %d)", ks, WAVE);
   IFX_REQUIRE(ch * ks >= d && ch * ks <= MAX_DPAD, "delta_rule: %d x %d channels for heads of %d (at most %d)", ch, ks, d, MAX_DPAD);
-  IFX_REQUIRE(dv <= MAX_DV && (long long)dv * ks <= 1024, "delta_rule: %d columns x %d threads do not fit a workgroup", dv, ks);
+  IFX_REQUIRE(cols > 0 && cols <= MAX_COLS && cols * ks <= 256, "delta_rule: %d columns x %d threads do not fit a workgroup of 256", cols, ks);
+  IFX_REQUIRE(STAGE * ch * ks <= MAX_PRE * 64 * ((cols * ks + 63) / 64) && STAGE * cols <= MAX_PRE * 64 * ((cols * ks + 63) / 64),
+              "delta_rule: a stage of %d x %d channels and %d columns is more than its %d threads fetch", STAGE, ch * ks, cols, cols * ks);
+  IFX_REQUIRE(T >= 0 && o_raw, "delta_rule: the read-outs need a place");
   IFX_REQUIRE(ldu >= 2 * G * d + H * dv && col_g >= 0 && col_b >= 0 && col_a >= 0, "delta_rule: rows too narrow");
   IFX_REQUIRE(state_stride >= state_offset + (long long)H * dv * ch * ks, "delta_rule: a state row of %lld floats is too short", state_stride);
   IFX_REQUIRE(R <= 65535, "delta_rule: too many requests for one launch");
   if (R == 0) return 0;
   DeltaArgs a{u, ldu, rows, ldr, col_g, col_b, col_a, A_log, dt_bias, norm_w, norm_dtype, eps, state, (size_t)state_stride,
-              (size_t)state_offset, q_start, q_len, slots, out, H, G, d, dv, ks};
-  const int threads = (dv * ks + WAVE - 1) / WAVE * WAVE;
-  const dim3 grid(H, R);
+              (size_t)state_offset, q_start, q_len, slots, out, o_raw, T, H, G, d, dv, ks, cols};
+  const int threads = (cols * ks + WAVE - 1) / WAVE * WAVE;
+  const dim3 grid(H * ((dv + cols - 1) / cols), R);
   hipStream_t s = (hipStream_t)stream;
 #define LAUNCH(TY, C) hipLaunchKernelGGL((delta_kernel<TY, C>), grid, dim3(threads), 0, s, a)
 #define BY_CH(TY)                                             \
@@ -170,5 +267,10 @@ extern "C" int ifx_delta_rule(const void* u, int ldu, const void* rows, int ldr,
   else IFX_FAIL("delta_rule: unknown dtype %d", dtype);
 #undef BY_CH
 #undef LAUNCH
+  if (T > 0) {
+    const unsigned blocks = (unsigned)(((size_t)T * H + 256 / WAVE - 1) / (256 / WAVE));
+    if (dtype == DT_F32) hipLaunchKernelGGL(delta_finish_kernel<float>, dim3(blocks), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(delta_finish_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, a);
+  }
   IFX_LAUNCH_CHECK();
 }

@@ -7,6 +7,10 @@
 //   scale_softcap  x <- cap * tanh(x * scale / cap) in place on float rows (cap 0: x <- x * scale)
 //   stream_add     x[t, c] <- x[t, c] + rows[t, c] + vec[c] in place on the float stream: what a pass of a looped span of
 //                  layers feeds into the stream before its first layer (either operand may be absent)
+//   diff_expand    q [T][H][2 d] -> [T][2 H][2 d]: head 2 h holds [q1 | 0] and head 2 h + 1 holds [0 | q2], so that attention
+//                  kernels for heads of 2 d elements score each half against its half of the keys' rows [k1 | k2]
+//   diff_combine   out[t, h, :] = o / sqrt(mean(o^2) + eps) * out_scale with o = a[t, 2 h, :] - lambda a[t, 2 h + 1, :]: the two
+//                  maps of differential attention joined, a wave per (row, head)
 // All arithmetic is float.
 #include "common.h"
 
@@ -192,5 +196,58 @@ extern "C" int ifx_stream_add(float* x, const float* rows, const void* vec, int 
   if (T == 0 || (!rows && !vec)) return 0;
   const size_t n = (size_t)T * H;
   hipLaunchKernelGGL(stream_add_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, x, rows, vec, vec_dtype, H, n);
+  IFX_LAUNCH_CHECK();
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void diff_expand_kernel(const T* __restrict__ q, T* __restrict__ out, int d, size_t n) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;        // an element of out
+  if (i >= n) return;
+  const int e = (int)(i % (2 * d));
+  const size_t head2 = i / (2 * d);                               // (row, head, map)
+  const int map = (int)(head2 & 1);
+  out[i] = (e >= d) == (map == 1) ? q[(head2 >> 1) * 2 * d + e] : from_f<T>(0.f);
+}
+
+extern "C" int ifx_diff_expand(const void* q, void* out, int dtype, long long rows_heads, int d, void* stream) {
+  IFX_REQUIRE(rows_heads >= 0 && d > 0, "diff_expand: bad sizes");
+  const size_t n = (size_t)rows_heads * 4 * d;
+  if (n == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  if (dtype == DT_BF16) hipLaunchKernelGGL(diff_expand_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, (const bf16_t*)q, (bf16_t*)out, d, n);
+  else if (dtype == DT_F32) hipLaunchKernelGGL(diff_expand_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)q, (float*)out, d, n);
+  else IFX_FAIL("diff_expand: unknown dtype %d", dtype);
+  IFX_LAUNCH_CHECK();
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void diff_combine_kernel(const T* __restrict__ a, T* __restrict__ out, size_t items, int dv, float lambda,
+                                                           float out_scale, float eps) {
+  const size_t item = (size_t)blockIdx.x * (256 / WAVE) + threadIdx.x / WAVE;       // (row, head)
+  const int lane = threadIdx.x % WAVE;
+  if (item >= items) return;
+  const T* a1 = a + item * 2 * dv;
+  const T* a2 = a1 + dv;
+  float ss = 0.f;
+  for (int c = lane; c < dv; c += WAVE) {
+    const float o = to_f(a1[c]) - lambda * to_f(a2[c]);
+    ss = fmaf(o, o, ss);
+  }
+  const float f = out_scale / sqrtf(wave_sum(ss) / (float)dv + eps);
+  for (int c = lane; c < dv; c += WAVE) out[item * dv + c] = from_f<T>((to_f(a1[c]) - lambda * to_f(a2[c])) * f);
+}
+
+extern "C" int ifx_diff_combine(const void* a, void* out, int dtype, long long rows_heads, int dv, float lambda, float out_scale, float eps,
+                                void* stream) {
+  IFX_REQUIRE(rows_heads >= 0 && dv > 0, "diff_combine: bad sizes");
+  if (rows_heads == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const unsigned blocks = (unsigned)((rows_heads + 256 / WAVE - 1) / (256 / WAVE));
+  if (dtype == DT_BF16)
+    hipLaunchKernelGGL(diff_combine_kernel<bf16_t>, dim3(blocks), dim3(256), 0, s, (const bf16_t*)a, (bf16_t*)out, (size_t)rows_heads, dv, lambda, out_scale, eps);
+  else if (dtype == DT_F32)
+    hipLaunchKernelGGL(diff_combine_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)a, (float*)out, (size_t)rows_heads, dv, lambda, out_scale, eps);
+  else IFX_FAIL("diff_combine: unknown dtype %d", dtype);
   IFX_LAUNCH_CHECK();
 }

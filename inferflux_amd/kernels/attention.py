@@ -225,15 +225,16 @@ def row_launch_shape(n_rows: int, n_kv_heads: int, max_kv: int, max_waves: int =
 
 def paged_attention(q: torch.Tensor, cache, ctx, window: Optional[int], scale: float, keep_first: int = 0,
                     sink: Optional[float] = None, gate: Optional[torch.Tensor] = None,
-                    sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    sinks: Optional[torch.Tensor] = None, block: Optional[int] = None) -> torch.Tensor:
     """q [T, nH, d] of this step's rows against ``cache`` (a LayerCache); returns [T, nH*d].  ``keep_first``: the first
     positions a windowed query sees beside its window; ``sink``: the score of a key without value in the softmax's
     denominator (None: none), ``sinks`` float32 [nH]: such a score for every head; ``gate`` float32
-    [T, nH]: a factor on every head's output."""
+    [T, nH]: a factor on every head's output; ``block``: a row sees only the keys of its own block of that many positions,
+    counted from the sequence's start."""
     T, nH, d = q.shape
     table = ctx.block_table(cache.group)
     keep_first = int(keep_first or 0) if window else 0
-    extras = keep_first > 0 or sink is not None or gate is not None or sinks is not None
+    extras = keep_first > 0 or sink is not None or gate is not None or sinks is not None or bool(block)
     if not ops.mfma_attention_supported(q.dtype, d, cache.page_size) or cache.v.shape[2] != d:
         # values of another width than the keys, or heads wider than a wave's registers hold: one shared kv head (attention
         # through a latent) has a matrix-core kernel of its own, everything else (32-bit, odd sizes) the plain kernel
@@ -241,7 +242,7 @@ def paged_attention(q: torch.Tensor, cache, ctx, window: Optional[int], scale: f
             chunk, splits = ops.wide_launch_shape(T, nH, ctx.kv_bound)
             return ops.attention_wide(q, cache.k, cache.v, ctx.row_req, ctx.positions, table, window, scale, chunk, splits)
         return ops.attention_plain(q, cache.k, cache.v, ctx.row_req, ctx.positions, table, window, scale, keep_first, sink, gate,
-                                   sinks=sinks)
+                                   sinks=sinks, chunk=block)
     n_kv = cache.k.shape[1]
     # Two query tiles per wave (128 rows per workgroup) read every key and value from LDS half as often.
     tiled = ctx.h_q_len >= TILE_MIN
@@ -253,7 +254,7 @@ def paged_attention(q: torch.Tensor, cache, ctx, window: Optional[int], scale: f
     w = ctx.derived(("attention_work_lists", n_kv, tile_rows, nH, splits, chunk, window, d),
                     lambda: _work_lists(ctx, n_kv, tile_rows, nH, splits, chunk, window, ops.row_waves_fit(nH, n_kv, d, ops.ROW_MAX_WAVES)))
     out = torch.empty((T, nH * d), dtype=q.dtype, device=q.device)
-    more = dict(keep_first=keep_first, sink=sink, gate=gate, sinks=sinks) if extras else {}
+    more = dict(keep_first=keep_first, sink=sink, gate=gate, sinks=sinks, block=block) if extras else {}
     if w["n_tiles"]:
         ops.attention_tiles(q, cache.k, cache.v, out, w["tile_req"], w["tile_q0"], ctx.q_start, ctx.q_len, ctx.kv_len,
                             table, window, scale, qt, w["tile_chunk"], w["tile_splits"], w["tile_row_list"], ctx.row_req,

@@ -1117,25 +1117,30 @@ def attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 
 # ----------------------------------------------------------------------------------------
 DELTA_THREAD_CHANNELS = (8, 16, 32, 64)     # key channels of a column of S a thread may hold
-DELTA_MAX_PADDED_DIM, DELTA_MAX_V_DIM = 256, 512
+DELTA_MAX_PADDED_DIM, DELTA_MAX_COLS, DELTA_THREADS = 256, 128, 256
 
 
-def delta_layout(d: int, dv: int) -> Tuple[int, int]:
-    """(channels a thread, threads a column) of the delta rule's kernel for heads of ``d`` key channels and ``dv`` values:
-    the fewest channels a thread whose columns still fit a workgroup of 1,024 threads (the threads of a column are a
-    power of two of neighbouring lanes)."""
+def delta_layout(d: int, dv: int) -> Tuple[int, int, int]:
+    """(channels a thread, threads a column, columns a workgroup) of the delta rule's kernel for heads of ``d`` key channels
+    and ``dv`` values: the fewest channels a thread (the threads of a column are a power of two of neighbouring lanes), and
+    as many columns as then fill a workgroup of 256 threads; a head's columns are dealt to as many workgroups as that takes.
+    The workgroup's threads must be at least the padded channels (each fetches its share of a stage of tokens)."""
     for ch in DELTA_THREAD_CHANNELS:
         ks = 1
         while ks * ch < d:
             ks *= 2
-        if ks <= 64 and ks * ch <= DELTA_MAX_PADDED_DIM and dv * ks <= 1024 and dv <= DELTA_MAX_V_DIM:
-            return ch, ks
+        if ks > 64 or ks * ch > DELTA_MAX_PADDED_DIM:
+            continue
+        cols = max(1, min(dv, DELTA_THREADS // ks, DELTA_MAX_COLS))
+        threads = -(-cols * ks // 64) * 64
+        if ch * ks <= threads:
+            return ch, ks, cols
     raise KernelError(f"delta rule: heads of {d} key channels and {dv} values fit no layout of the kernel (at most "
-                      f"{DELTA_MAX_PADDED_DIM} channels, {DELTA_MAX_V_DIM} values, and columns x threads a column within 1,024)")
+                      f"{DELTA_MAX_PADDED_DIM} channels, and no more of them than a workgroup's columns have threads)")
 
 
 def delta_state_floats(n_heads: int, d: int, dv: int) -> int:
-    ch, ks = delta_layout(d, dv)
+    ch, ks, _ = delta_layout(d, dv)
     return n_heads * dv * ch * ks
 
 
@@ -1162,14 +1167,38 @@ def delta_rule(u: torch.Tensor, rows: torch.Tensor, cols: Tuple[int, int, int], 
     R = q_start.shape[0]
     for t, nm in ((q_start, "q_start"), (q_len, "q_len"), (slots, "slots")):
         _check(t, nm, (R,), torch.int32)
-    ch, ks = delta_layout(d, dv)
+    ch, ks, cols = delta_layout(d, dv)
     if state_offset + H * dv * ch * ks > state.shape[1]:
         raise KernelError("delta_rule: the state rows are too short")
     out = torch.empty((T, H * dv), dtype=u.dtype, device=u.device)
-    _call(load_module("delta"), "ifx_delta_rule", (P, I, P, I, I, I, I, I, P, P, P, I, F, P, LL, LL, P, P, P, P, I, I, I, I, I, I, I, P),
+    o_raw = torch.empty((T, H * dv), dtype=torch.float32, device=u.device)
+    _call(load_module("delta"), "ifx_delta_rule", (P, I, P, I, I, I, I, I, P, P, P, I, F, P, LL, LL, P, P, P, P, P, I, I, I, I, I, I, I, I, I, P),
           u.data_ptr(), ldu, rows.data_ptr(), ldr, col_g, col_b, col_a, _dt(u), A_log.data_ptr(), dt_bias.data_ptr(),
           norm_w.data_ptr(), _dt(norm_w), float(eps), state.data_ptr(), state.shape[1], int(state_offset), q_start.data_ptr(),
-          q_len.data_ptr(), slots.data_ptr(), out.data_ptr(), R, H, G, d, dv, ch, ks, _stream())
+          q_len.data_ptr(), slots.data_ptr(), out.data_ptr(), o_raw.data_ptr(), T, R, H, G, d, dv, ch, ks, cols, _stream())
+    return out
+
+
+def diff_expand(q: torch.Tensor) -> torch.Tensor:
+    """q [T, H, 2 d] -> [T, 2 H, 2 d]: head 2 h is [q1 | 0], head 2 h + 1 is [0 | q2] (the two maps of differential attention as
+    heads of their own against keys whose rows hold both maps' vectors)."""
+    _check(q, "q", (None, None, None))
+    T, H, two_d = q.shape
+    if two_d % 2:
+        raise KernelError("diff_expand: a row of two maps has an even number of elements")
+    out = torch.empty((T, 2 * H, two_d), dtype=q.dtype, device=q.device)
+    _call(load_module("rowwise"), "ifx_diff_expand", (P, P, I, LL, I, P), q.data_ptr(), out.data_ptr(), _dt(q), T * H, two_d // 2, _stream())
+    return out
+
+
+def diff_combine(a: torch.Tensor, n_heads: int, dv: int, lam: float, out_scale: float, eps: float) -> torch.Tensor:
+    """a [T, 2 H dv] (per head the two maps' outputs, one after the other) -> [T, H dv]: o = a1 - lam a2, divided by its root
+    mean square over dv (eps inside the root), times out_scale."""
+    _check(a, "a", (None, 2 * n_heads * dv))
+    T = a.shape[0]
+    out = torch.empty((T, n_heads * dv), dtype=a.dtype, device=a.device)
+    _call(load_module("rowwise"), "ifx_diff_combine", (P, P, I, LL, I, F, F, F, P), a.data_ptr(), out.data_ptr(), _dt(a), T * n_heads, dv,
+          float(lam), float(out_scale), float(eps), _stream())
     return out
 
 
@@ -1548,14 +1577,14 @@ def _attn_common(q, k_cache, v_cache, qt=1, direct=True):
     return T, nH, d, nKV, page_size, load_module(name, variant)
 
 
-def _attn_extras(T, nH, keep_first, sink, gate, sinks=None):
-    """The five optional arguments of the matrix-core attention kernels: kept first keys, whether there is a sink, its
-    score, the gate's pointer, the pointer to a sink score per head."""
+def _attn_extras(T, nH, keep_first, sink, gate, sinks=None, block=None):
+    """The six optional arguments of the matrix-core attention kernels: kept first keys, whether there is a sink, its
+    score, the gate's pointer, the pointer to a sink score per head, the size of the blocks a row sees its own of."""
     if gate is not None:
         _check(gate, "gate", (T, nH), torch.float32)
     if sinks is not None:
         _check(sinks, "sinks", (nH,), torch.float32)
-    return int(keep_first or 0), 0 if sink is None else 1, float(sink or 0.0), _ptr(gate), _ptr(sinks)
+    return int(keep_first or 0), 0 if sink is None else 1, float(sink or 0.0), _ptr(gate), _ptr(sinks), int(block or 0)
 
 
 ROW_MAX_WAVES = 8
@@ -1573,7 +1602,7 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
                    rows: Optional[torch.Tensor], n_rows: int, row_req: torch.Tensor, positions: torch.Tensor,
                    block_table: torch.Tensor, window: Optional[int], scale: float, chunk: int, max_splits: int,
                    waves: int = 0, req_is_row: bool = False, keep_first: int = 0, sink: Optional[float] = None,
-                   gate: Optional[torch.Tensor] = None, sinks: Optional[torch.Tensor] = None) -> None:
+                   gate: Optional[torch.Tensor] = None, sinks: Optional[torch.Tensor] = None, block: Optional[int] = None) -> None:
     """Attention of single rows (``rows`` int32, or None for rows 0..n_rows-1) into ``out`` [T, nH*d].  ``keep_first``,
     ``sink``, ``gate``: as for ``attention_plain``.
 
@@ -1601,11 +1630,11 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         part_ml = torch.empty((n_rows, nH, max_splits, 2), dtype=torch.float32, device=q.device)
     if req_is_row and block_table.shape[0] < T:
         raise KernelError("attention_rows: req_is_row needs a block-table row for every row of the step")
-    _call(mod, "ifx_attn_rows", (P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, P, P, I, I, I, I, F, P, P, P),
+    _call(mod, "ifx_attn_rows", (P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, P, P, I, I, I, I, F, P, P, I, P),
           q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _ptr(rows), row_req.data_ptr(),
           positions.data_ptr(), block_table.data_ptr(), block_table.shape[1], n_rows, nH, nKV, d, page_size,
           int(window or 0), chunk, max_splits, float(scale), _ptr(part_o), _ptr(part_ml), waves, 1 if req_is_row else 0,
-          *_attn_extras(T, nH, keep_first, sink, gate, sinks), _stream())
+          *_attn_extras(T, nH, keep_first, sink, gate, sinks, block), _stream())
 
 
 def attention_tile_rows(head_dim: int, qt: int = 1) -> int:
@@ -1620,7 +1649,7 @@ def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                     qt: int = 1, chunk: int = 0, max_splits: int = 1, rows: Optional[torch.Tensor] = None,
                     row_req: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None,
                     order: Optional[torch.Tensor] = None, keep_first: int = 0, sink: Optional[float] = None,
-                    gate: Optional[torch.Tensor] = None, sinks: Optional[torch.Tensor] = None) -> None:
+                    gate: Optional[torch.Tensor] = None, sinks: Optional[torch.Tensor] = None, block: Optional[int] = None) -> None:
     """Attention of tiles of ``attention_tile_rows(d, qt)`` consecutive rows of one request each (tile t:
     request tile_req[t], rows from tile_q0[t] of that request's rows in this step) into ``out`` [T, nH*d].
 
@@ -1631,7 +1660,7 @@ def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 
     ``order`` (int32 [8 * n], from ``attention.tile_order``) says which work item each workgroup of the launch
     takes; every item must appear exactly once (-1: a workgroup without work).  The result does not depend on it."""
-    extras = bool(keep_first) or sink is not None or gate is not None or sinks is not None      # (the kernel that loads straight into LDS has none of them)
+    extras = bool(keep_first) or sink is not None or gate is not None or sinks is not None or bool(block)      # (the kernel that loads straight into LDS has none of them)
     T, nH, d, nKV, page_size, mod = _attn_common(q, k_cache, v_cache, qt, not extras)
     _, _, entry, rows_fn = _tile_module(d, qt, not extras)
     if mod.fn(rows_fn, ())() != attention_tile_rows(d, qt):
@@ -1669,7 +1698,7 @@ def attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             _ptr(part_o), _ptr(part_ml), _ptr(rows), n_rows, _ptr(row_req), _ptr(positions), _ptr(order), per_xcd, N_XCD)
     types = (P, P, P, P, P, P, I, P, P, P, P, I, I, I, I, I, I, F, I, I, P, P, P, I, P, P, P, I, I)
     if entry == "ifx_attn_tiles":
-        _call(mod, entry, types + (I, I, F, P, P, P), *args, *_attn_extras(T, nH, keep_first, sink, gate, sinks), _stream())
+        _call(mod, entry, types + (I, I, F, P, P, I, P), *args, *_attn_extras(T, nH, keep_first, sink, gate, sinks, block), _stream())
     else:
         _call(mod, entry, types + (P,), *args, _stream())
 

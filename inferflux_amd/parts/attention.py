@@ -191,12 +191,19 @@ class PagedAttention(Mixer):
         return ops.linear(out, self.w_o, keep_slices=sink is not None)   # an RMS norm's kernel adds partial sums itself
 
     def _attend(self, q, cache, ctx, gate=None):
-        if self.chunk is not None or self.differential is not None:
-            # the kernel that knows blocks and two maps: one wave per (row, head), float or bfloat16 storage, float math
-            diff = None if self.differential is None else (self.lam, 1.0 - self.differential[0], self.differential[1])
-            return ops.attention_plain(q, cache.k, cache.v, ctx.row_req, ctx.positions, ctx.block_table(cache.group), self.window,
-                                       self.scale, self.keep_first, self.sink, gate, chunk=self.chunk, differential=diff)
-        return paged_attention(q, cache, ctx, self.window, self.scale, self.keep_first, self.sink, gate)
+        if self.differential is None:
+            return paged_attention(q, cache, ctx, self.window, self.scale, self.keep_first, self.sink, gate, block=self.chunk)
+        lam, out_scale, eps = self.lam, 1.0 - self.differential[0], self.differential[1]
+        if (self.v_head_dim == self.head_dim and gate is None and self.sink is None and not self.keep_first
+                and ops.mfma_attention_supported(q.dtype, self.head_dim, cache.page_size)):
+            # Values as wide as both maps' keys together: each map becomes a head of its own whose query is padded with
+            # zeros over the other map's half, which the matrix-core kernels score against the keys' whole rows; a small
+            # kernel joins the two outputs.
+            a = paged_attention(ops.diff_expand(q), cache, ctx, self.window, self.scale, block=self.chunk)
+            return ops.diff_combine(a, self.n_heads, self.v_head_dim, lam, out_scale, eps)
+        # any other sizes, and 32-bit: the kernel that knows two maps, one wave per (row, head), float math
+        return ops.attention_plain(q, cache.k, cache.v, ctx.row_req, ctx.positions, ctx.block_table(cache.group), self.window,
+                                   self.scale, self.keep_first, self.sink, gate, chunk=self.chunk, differential=(lam, out_scale, eps))
 
     def _forward_extras(self, h, ctx, binding: MixerBinding, sink):
         """The step with the optional mechanisms: the fused projection (with the gate's rows), one row kernel for bias,

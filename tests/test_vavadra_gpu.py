@@ -331,7 +331,44 @@ def test_a_pass_input_is_added_to_the_stream_in_place():
             assert rel_err(got, want) < 1e-6
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_two_maps_as_heads_of_their_own_and_joined_again(dtype):
+    dt, T, H, d, dv = DT[dtype], 37, 3, 16, 32
+    q = rnd(1, T, H, 2 * d).to(dt)
+    wide = ops.diff_expand(q.to(DEV)).cpu()
+    assert wide.shape == (T, 2 * H, 2 * d)
+    assert torch.equal(wide[:, 0::2, :d], q[:, :, :d]) and torch.equal(wide[:, 1::2, d:], q[:, :, d:])
+    assert float(wide[:, 0::2, d:].abs().max()) == 0 and float(wide[:, 1::2, :d].abs().max()) == 0
+    a = rnd(2, T, 2 * H * dv).to(dt)
+    lam, scale, eps = 0.63, 0.7, 1e-5
+    pairs = N64(a).reshape(T, H, 2, dv)
+    want = pv.rms_norm(pairs[:, :, 0] - lam * pairs[:, :, 1], None, eps) * scale
+    got = ops.diff_combine(a.to(DEV), H, dv, lam, scale, eps).cpu()
+    assert rel_err(got, T64(want.reshape(T, H * dv))) < (1e-6 if dtype == "float32" else 1e-2)
+
+
 # ---- the model through the engine -----------------------------------------------------------------
+@pytest.mark.parametrize("chunk", [17, 48, 100, 64, None])
+def test_blocks_and_two_maps_on_the_matrix_cores(chunk, tmp_path):
+    """Differential attention whose values are as wide as both maps' keys together runs on the matrix-core kernels in bfloat16:
+    blocks whose edges lie inside the kernels' tiles of keys and of rows, in a prompt, in portions and token by token."""
+    cfg = vm.model(200, 64, 1e-5, [vm.layer(vm.differential(4, 2, 32, 64, 0.2, 0.4, chunk=chunk), None),
+                                   vm.layer(vm.differential(2, 2, 8, 16, 0.4, 0.7, chunk=chunk), vm.moe(4, 1, 2, 16, 2.0))], emb_scale=2.0)
+    folder = vm.write_model(str(tmp_path / "m"), cfg, 3, gain=1.5, decisive_router=True)
+    runner = load_runner(folder, torch.bfloat16, num_pages=40, max_requests=3)
+    ids = ids_of(5, 330, 200)
+    want = plain(folder, ids)
+    assert off(run_whole(runner, "w", ids), want, "bfloat16") < 1
+    runner.add_request("c")
+    rows, p = [], 0
+    for m in [100, 1, 1, 63, 2, 17, 1, 1, 1, 1, 130, 2, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1]:
+        rows.append(runner.step([StepEntry("c", ids[p:p + m], list(range(m)))]).cpu())
+        p += m
+    assert p == len(ids) and off(torch.cat(rows), want, "bfloat16") < 1
+    runner.manager.check()
+
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", list(vm.CONFIGS))
 def test_whole_prompts(name, dtype, folders):
