@@ -134,7 +134,7 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(2, 2))) vo
   l = col_sum(l);
   if (!head_ok) return;
   if (a.max_splits == 1) {      // the row's only split: the output itself, no partial result and no merge
-    const float inv = l > 0.f ? 1.f / l : 0.f;
+    const float inv = finish_factor(m, l, 0, 0.f, nullptr, (size_t)row * a.nH + head, a.sinks, a.nH);      // (a sink score per head joins the sum here)
     bf16_t* orow = a.out + ((size_t)row * a.nH + head) * D;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
@@ -180,7 +180,7 @@ __global__ __launch_bounds__(WAVE) void attn_wide_merge_kernel(RowArgs a) {
       }
     }
   }
-  const float inv = L > 0.f ? 1.f / L : 0.f;
+  const float inv = finish_factor(M, L, 0, 0.f, nullptr, (size_t)row * a.nH + head, a.sinks, a.nH);
   bf16_t* orow = a.out + ((size_t)row * a.nH + head) * D;
 #pragma unroll
   for (int c = 0; c < C4; ++c) {
@@ -200,7 +200,7 @@ __global__ __launch_bounds__(WAVE) void attn_wide_merge_kernel(RowArgs a) {
 extern "C" int ifx_attn_wide(const void* q, const void* k_cache, const void* v_cache, void* out, const int* rows,
                              const int* row_req, const int* positions, const int* block_table, int max_blocks, int n_rows,
                              int nH, int d, int dv, int page_size, int window, int chunk, int max_splits, float scale,
-                             float* part_o, float* part_ml, void* stream) {
+                             float* part_o, float* part_ml, const float* sinks, void* stream) {
   IFX_REQUIRE(d == DK && dv == D, "attn_wide: built for keys of %d and values of %d, called with %d and %d", DK, D, d, dv);
   IFX_REQUIRE(n_rows >= 0 && n_rows <= 65535 && nH > 0 && (nH + 15) / 16 <= 65535, "attn_wide: %d rows, %d heads", n_rows, nH);
   IFX_REQUIRE(page_size >= 16 && page_size % 16 == 0, "attn_wide: page_size %d must be a multiple of 16", page_size);
@@ -210,6 +210,7 @@ extern "C" int ifx_attn_wide(const void* q, const void* k_cache, const void* v_c
   RowArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, rows, row_req, positions, block_table,
             part_o, part_ml, (bf16_t*)out, max_blocks, n_rows, nH, 1, page_size, window, chunk, max_splits,
             scale * 1.4426950408889634f, 0, 0, 0};
+  a.sinks = sinks;          // [nH] or null: a score per head in the softmax's denominator
   hipStream_t s = (hipStream_t)stream;
   hipLaunchKernelGGL(attn_wide_rows_kernel, dim3(max_splits, (nH + 15) / 16, n_rows), dim3(WAVE), (size_t)16 * QP * sizeof(bf16_t), s, a);
   if (max_splits > 1) hipLaunchKernelGGL(attn_wide_merge_kernel, dim3(n_rows, nH), dim3(WAVE), 0, s, a);

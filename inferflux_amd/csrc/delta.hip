@@ -51,7 +51,9 @@ __device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log
 #define STAGE 16
 #define MAX_DPAD 256
 #define MAX_COLS 128
-#define MAX_PRE 16          // 16-byte-free prefetch: values a thread holds for the next stage (see below)
+#define MAX_PRE 16          // q and k elements of a stage a thread fetches at most (STAGE * d_pad / threads)
+#define MAX_PRE_V 8         // ... and v elements (STAGE * columns / threads)
+//          // 16-byte-free prefetch: values a thread holds for the next stage (see below)
 
 // The sum over the KS (a power of two) neighbouring lanes that share a column, in every one of them: neighbours within a
 // row of 16 lanes swap through the lanes' own data paths (pairs, quads, mirrored halves of 8, mirrored rows of 16: a few
@@ -74,8 +76,9 @@ __device__ __forceinline__ float column_sum(float v, int KS) {
 
 template <typename T, int CH>
 __global__ __launch_bounds__(256) void delta_kernel(DeltaArgs a) {
-  __shared__ float q_s[STAGE][MAX_DPAD], k_s[STAGE][MAX_DPAD];
-  __shared__ float v_s[STAGE][MAX_COLS], o_s[STAGE][MAX_COLS];
+  // LDS as the head's sizes need it (so that several workgroups share a compute unit): q and k of a stage [STAGE][dpad]
+  // each, then its v and o [STAGE][cols] each
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   __shared__ float beta_s[STAGE], g_s[STAGE];
   const int n_cb = (a.dv + a.cols - 1) / a.cols;
   const int h = blockIdx.x / n_cb, j0 = (blockIdx.x % n_cb) * a.cols, r = blockIdx.y;
@@ -84,6 +87,10 @@ __global__ __launch_bounds__(256) void delta_kernel(DeltaArgs a) {
   const int t0 = a.q_start[r];
   const int d = a.d, dv = a.dv, KS = a.KS, dpad = CH * KS;
   const int cols = min(a.cols, dv - j0);
+  float* q_s = lds;
+  float* k_s = lds + STAGE * dpad;
+  float* v_s = lds + 2 * STAGE * dpad;
+  float* o_s = v_s + STAGE * a.cols;
   const int g = h / (a.H / a.G);
   const int tid = threadIdx.x, nthr = blockDim.x;
   const int wid = tid / WAVE, lane = tid % WAVE, nw = (nthr + WAVE - 1) / WAVE;
@@ -102,14 +109,10 @@ __global__ __launch_bounds__(256) void delta_kernel(DeltaArgs a) {
   // (dpad is a power of two; the places of a thread's v elements are the same in every stage and found once)
   const int per_qk = (STAGE * dpad + nthr - 1) / nthr, per_v = (STAGE * cols + nthr - 1) / nthr;
   const int dshift = __ffs(dpad) - 1;
-  int v_tt[MAX_PRE], v_c[MAX_PRE];
-#pragma unroll
-  for (int e = 0; e < MAX_PRE; ++e) {
-    const int x = tid + e * nthr;
-    v_tt[e] = e < per_v ? x / cols : STAGE;
-    v_c[e] = e < per_v ? x % cols : 0;
-  }
-  float pq[MAX_PRE], pk[MAX_PRE], pv[MAX_PRE], pb = 0.f, pg = 0.f;
+  // a thread's v elements of a stage are x = tid, tid + nthr, ...: (token, column) = (x / cols, x % cols), stepped from the
+  // first by (nthr / cols, nthr % cols) with a carry, so that one division a thread is all there is
+  const int v_tt0 = tid / cols, v_c0 = tid - v_tt0 * cols, v_dq = nthr / cols, v_dr = nthr - v_dq * cols;
+  float pq[MAX_PRE], pk[MAX_PRE], pv[MAX_PRE_V], pb = 0.f, pg = 0.f;
   auto fetch = [&](int base) {
     const int cnt = min(STAGE, n - base);
 #pragma unroll
@@ -121,12 +124,14 @@ __global__ __launch_bounds__(256) void delta_kernel(DeltaArgs a) {
       pq[e] = in ? to_f(u[row + (size_t)g * d + c]) : 0.f;
       pk[e] = in ? to_f(u[row + (size_t)(a.G + g) * d + c]) : 0.f;
     }
+    int tt = v_tt0, c = v_c0;
 #pragma unroll
-    for (int e = 0; e < MAX_PRE; ++e) {
+    for (int e = 0; e < MAX_PRE_V; ++e) {
       if (e >= per_v) break;
-      const int tt = v_tt[e], c = v_c[e];
       const bool in = tt < cnt;
       pv[e] = in ? to_f(u[(size_t)(t0 + base + tt) * a.ldu + (size_t)2 * a.G * d + (size_t)h * dv + j0 + c]) : 0.f;
+      tt += v_dq; c += v_dr;
+      if (c >= cols) { c -= cols; ++tt; }
     }
     if (tid < cnt) {
       const size_t row = (size_t)(t0 + base + tid) * a.ldr;
@@ -142,12 +147,17 @@ __global__ __launch_bounds__(256) void delta_kernel(DeltaArgs a) {
     for (int e = 0; e < MAX_PRE; ++e) {
       if (e >= per_qk) break;
       const int x = tid + e * nthr;
-      if (x < STAGE * dpad) { q_s[x >> dshift][x & (dpad - 1)] = pq[e]; k_s[x >> dshift][x & (dpad - 1)] = pk[e]; }
+      if (x < STAGE * dpad) { q_s[x] = pq[e]; k_s[x] = pk[e]; }
     }
+    {
+      int tt = v_tt0, c = v_c0;
 #pragma unroll
-    for (int e = 0; e < MAX_PRE; ++e) {
-      if (e >= per_v) break;
-      if (v_tt[e] < STAGE) v_s[v_tt[e]][v_c[e]] = pv[e];
+      for (int e = 0; e < MAX_PRE_V; ++e) {
+        if (e >= per_v) break;
+        if (tt < STAGE) v_s[tt * a.cols + c] = pv[e];
+        tt += v_dq; c += v_dr;
+        if (c >= cols) { c -= cols; ++tt; }
+      }
     }
     if (tid < cnt) {
       beta_s[tid] = 1.0f / (1.0f + expf(-pb));
@@ -158,7 +168,7 @@ __global__ __launch_bounds__(256) void delta_kernel(DeltaArgs a) {
     // unit norms: NL neighbouring lanes per (token, q or k), all pairs at once; the lanes' squares added by column_sum
     {
       const int pair = tid / NL, l = tid % NL;
-      float* vec = (pair & 1) ? k_s[min(pair >> 1, STAGE - 1)] : q_s[min(pair >> 1, STAGE - 1)];
+      float* vec = ((pair & 1) ? k_s : q_s) + min(pair >> 1, STAGE - 1) * dpad;
       const bool mine = pair < 2 * cnt;
       float ss = 0.f;
       if (mine)
@@ -173,18 +183,18 @@ __global__ __launch_bounds__(256) void delta_kernel(DeltaArgs a) {
     if (owner) {
       // a token's k, q, v, decay and beta are read from LDS while the token before it is worked on; the sums over a
       // thread's channels run in four chains that are added at the end (a fixed order)
-      float kn[CH], qn[CH], vn = v_s[0][jl], gn = g_s[0], bn = beta_s[0];
+      float kn[CH], qn[CH], vn = v_s[jl], gn = g_s[0], bn = beta_s[0];
 #pragma unroll
-      for (int i = 0; i < CH; ++i) { kn[i] = k_s[0][s * CH + i]; qn[i] = q_s[0][s * CH + i]; }
+      for (int i = 0; i < CH; ++i) { kn[i] = k_s[s * CH + i]; qn[i] = q_s[s * CH + i]; }
       for (int tt = 0; tt < cnt; ++tt) {
         float kk[CH], qq[CH];
         const float gd = gn, bt = bn, vt = vn;
 #pragma unroll
         for (int i = 0; i < CH; ++i) { kk[i] = kn[i]; qq[i] = qn[i]; }
         if (tt + 1 < cnt) {
-          vn = v_s[tt + 1][jl]; gn = g_s[tt + 1]; bn = beta_s[tt + 1];
+          vn = v_s[(tt + 1) * a.cols + jl]; gn = g_s[tt + 1]; bn = beta_s[tt + 1];
 #pragma unroll
-          for (int i = 0; i < CH; ++i) { kn[i] = k_s[tt + 1][s * CH + i]; qn[i] = q_s[tt + 1][s * CH + i]; }
+          for (int i = 0; i < CH; ++i) { kn[i] = k_s[(tt + 1) * dpad + s * CH + i]; qn[i] = q_s[(tt + 1) * dpad + s * CH + i]; }
         }
         float p4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -201,12 +211,12 @@ __global__ __launch_bounds__(256) void delta_kernel(DeltaArgs a) {
           o4[i & 3] = fmaf(S[i], qq[i], o4[i & 3]);
         }
         const float out = column_sum((o4[0] + o4[1]) + (o4[2] + o4[3]), KS);
-        if (s == 0) o_s[tt][jl] = out;
+        if (s == 0) o_s[tt * a.cols + jl] = out;
       }
     }
     LDS_BARRIER();
     for (int x = tid; x < cnt * cols; x += nthr)
-      a.o_raw[((size_t)(t0 + base + x / cols) * a.H + h) * dv + j0 + x % cols] = o_s[x / cols][x % cols];
+      a.o_raw[((size_t)(t0 + base + x / cols) * a.H + h) * dv + j0 + x % cols] = o_s[(x / cols) * a.cols + x % cols];
   }
   if (owner) {
 #pragma unroll
@@ -241,7 +251,7 @@ extern "C" int ifx_delta_rule(const void* u, int ldu, const void* rows, int ldr,
   IFX_REQUIRE(ks > 0 && ks <= WAVE && (ks & (ks - 1)) == 0, "delta_rule: %d threads to a column (a power of two up to %d)", ks, WAVE);
   IFX_REQUIRE(ch * ks >= d && ch * ks <= MAX_DPAD, "delta_rule: %d x %d channels for heads of %d (at most %d)", ch, ks, d, MAX_DPAD);
   IFX_REQUIRE(cols > 0 && cols <= MAX_COLS && cols * ks <= 256, "delta_rule: %d columns x %d threads do not fit a workgroup of 256", cols, ks);
-  IFX_REQUIRE(STAGE * ch * ks <= MAX_PRE * 64 * ((cols * ks + 63) / 64) && STAGE * cols <= MAX_PRE * 64 * ((cols * ks + 63) / 64),
+  IFX_REQUIRE(STAGE * ch * ks <= MAX_PRE * 64 * ((cols * ks + 63) / 64) && STAGE * cols <= MAX_PRE_V * 64 * ((cols * ks + 63) / 64),
               "delta_rule: a stage of %d x %d channels and %d columns is more than its %d threads fetch", STAGE, ch * ks, cols, cols * ks);
   IFX_REQUIRE(T >= 0 && o_raw, "delta_rule: the read-outs need a place");
   IFX_REQUIRE(ldu >= 2 * G * d + H * dv && col_g >= 0 && col_b >= 0 && col_a >= 0, "delta_rule: rows too narrow");
@@ -253,14 +263,16 @@ extern "C" int ifx_delta_rule(const void* u, int ldu, const void* rows, int ldr,
   const int threads = (cols * ks + WAVE - 1) / WAVE * WAVE;
   const dim3 grid(H * ((dv + cols - 1) / cols), R);
   hipStream_t s = (hipStream_t)stream;
-#define LAUNCH(TY, C) hipLaunchKernelGGL((delta_kernel<TY, C>), grid, dim3(threads), 0, s, a)
+  const size_t lds_bytes = (size_t)2 * STAGE * (ch * ks + cols) * sizeof(float);
+#define LAUNCH(TY, C) hipLaunchKernelGGL((delta_kernel<TY, C>), grid, dim3(threads), lds_bytes, s, a)
 #define BY_CH(TY)                                             \
   do {                                                        \
-    if (ch == 8) LAUNCH(TY, 8);                               \
+    if (ch == 4) LAUNCH(TY, 4);                               \
+    else if (ch == 8) LAUNCH(TY, 8);                          \
     else if (ch == 16) LAUNCH(TY, 16);                        \
     else if (ch == 32) LAUNCH(TY, 32);                        \
     else if (ch == 64) LAUNCH(TY, 64);                        \
-    else IFX_FAIL("delta_rule: %d channels a thread (8, 16, 32 or 64)", ch); \
+    else IFX_FAIL("delta_rule: %d channels a thread (4, 8, 16, 32 or 64)", ch); \
   } while (0)
   if (dtype == DT_F32) BY_CH(float);
   else if (dtype == DT_BF16) BY_CH(bf16_t);

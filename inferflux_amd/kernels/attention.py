@@ -238,9 +238,10 @@ def paged_attention(q: torch.Tensor, cache, ctx, window: Optional[int], scale: f
     if not ops.mfma_attention_supported(q.dtype, d, cache.page_size) or cache.v.shape[2] != d:
         # values of another width than the keys, or heads wider than a wave's registers hold: one shared kv head (attention
         # through a latent) has a matrix-core kernel of its own, everything else (32-bit, odd sizes) the plain kernel
-        if not extras and ops.wide_attention_supported(q.dtype, cache.k.shape[1], d, cache.v.shape[2], cache.page_size):
+        other = keep_first > 0 or sink is not None or gate is not None or bool(block)      # (a sink score per head it does take)
+        if not other and ops.wide_attention_supported(q.dtype, cache.k.shape[1], d, cache.v.shape[2], cache.page_size):
             chunk, splits = ops.wide_launch_shape(T, nH, ctx.kv_bound)
-            return ops.attention_wide(q, cache.k, cache.v, ctx.row_req, ctx.positions, table, window, scale, chunk, splits)
+            return ops.attention_wide(q, cache.k, cache.v, ctx.row_req, ctx.positions, table, window, scale, chunk, splits, sinks)
         return ops.attention_plain(q, cache.k, cache.v, ctx.row_req, ctx.positions, table, window, scale, keep_first, sink, gate,
                                    sinks=sinks, chunk=block)
     n_kv = cache.k.shape[1]

@@ -1116,42 +1116,61 @@ def attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 
 
 # ----------------------------------------------------------------------------------------
-DELTA_THREAD_CHANNELS = (8, 16, 32, 64)     # key channels of a column of S a thread may hold
+DELTA_THREAD_CHANNELS = (4, 8, 16, 32, 64)  # key channels of a column of S a thread may hold
 DELTA_MAX_PADDED_DIM, DELTA_MAX_COLS, DELTA_THREADS = 256, 128, 256
+DELTA_DECODE_MAX_CHANNELS = 16              # ... at most this many in steps of single tokens (more would not fit the registers)
 
 
-def delta_layout(d: int, dv: int) -> Tuple[int, int, int]:
+def delta_padded_dim(d: int) -> int:
+    """The key channels of a head padded to a power of two (at least 4): what a column of S takes in a request's state."""
+    p = 4
+    while p < d:
+        p *= 2
+    if p > DELTA_MAX_PADDED_DIM:
+        raise KernelError(f"delta rule: heads of {d} key channels (at most {DELTA_MAX_PADDED_DIM})")
+    return p
+
+
+def delta_layout(d: int, dv: int, single_tokens: bool = False) -> Tuple[int, int, int]:
     """(channels a thread, threads a column, columns a workgroup) of the delta rule's kernel for heads of ``d`` key channels
-    and ``dv`` values: the fewest channels a thread (the threads of a column are a power of two of neighbouring lanes), and
-    as many columns as then fill a workgroup of 256 threads; a head's columns are dealt to as many workgroups as that takes.
-    The workgroup's threads must be at least the padded channels (each fetches its share of a stage of tokens)."""
+    and ``dv`` values.  The threads of a column are a power of two of neighbouring lanes that share the padded channels; a
+    workgroup has up to 256 threads and a head's columns are dealt to as many workgroups as that takes.  The state's layout
+    does not depend on the choice, so a step takes the one that suits it: a prompt's portion is a chain from token to token,
+    which is shortest with the fewest channels a thread; steps of single tokens are many short workgroups, of which there
+    should be few (``single_tokens``)."""
+    dpad = delta_padded_dim(d)
+    found = []
     for ch in DELTA_THREAD_CHANNELS:
-        ks = 1
-        while ks * ch < d:
-            ks *= 2
-        if ks > 64 or ks * ch > DELTA_MAX_PADDED_DIM:
+        if ch > dpad or dpad // ch > 64:
             continue
+        ks = dpad // ch
         cols = max(1, min(dv, DELTA_THREADS // ks, DELTA_MAX_COLS))
         threads = -(-cols * ks // 64) * 64
-        if ch * ks <= threads:
-            return ch, ks, cols
-    raise KernelError(f"delta rule: heads of {d} key channels and {dv} values fit no layout of the kernel (at most "
-                      f"{DELTA_MAX_PADDED_DIM} channels, and no more of them than a workgroup's columns have threads)")
+        if dpad <= threads and 2 * cols <= threads:         # (each thread fetches its share of a stage of sixteen tokens)
+            found.append((ch, ks, cols))
+    if not found:
+        raise KernelError(f"delta rule: heads of {d} key channels and {dv} values fit no layout of the kernel")
+    if single_tokens:
+        few = [f for f in found if f[0] <= DELTA_DECODE_MAX_CHANNELS] or found
+        return min(few, key=lambda f: (-(-dv // f[2]), f[0]))
+    return found[0]
 
 
 def delta_state_floats(n_heads: int, d: int, dv: int) -> int:
-    ch, ks, _ = delta_layout(d, dv)
-    return n_heads * dv * ch * ks
+    delta_layout(d, dv)
+    return n_heads * dv * delta_padded_dim(d)
 
 
 def delta_rule(u: torch.Tensor, rows: torch.Tensor, cols: Tuple[int, int, int], A_log: torch.Tensor, dt_bias: torch.Tensor,
                norm_w: torch.Tensor, eps: float, n_heads: int, n_kv_heads: int, d: int, dv: int, state: torch.Tensor,
-               state_offset: int, q_start: torch.Tensor, q_len: torch.Tensor, slots: torch.Tensor) -> torch.Tensor:
+               state_offset: int, q_start: torch.Tensor, q_len: torch.Tensor, slots: torch.Tensor,
+               single_tokens: bool = False) -> torch.Tensor:
     """The gated delta rule over a step's rows (see csrc/delta.hip).  ``u`` [T, >= 2 G d + H dv] holds per row the q heads,
     the k heads and the v heads (after their convolution), ``rows`` [T, ld] the gate's H dv columns from ``cols[0]``, beta's
     H from ``cols[1]`` and the decay's H from ``cols[2]``, both in the activation type.  ``A_log``, ``dt_bias`` float32 [H],
     ``norm_w`` [dv].  A request's S lies ``state_offset`` floats into its row of ``state`` [slots, n] (float32), zero for a
-    request that starts.  Returns [T, H dv] in u's type."""
+    request that starts.  ``single_tokens``: every request brings one row (the launch then takes few, larger workgroups).
+    Returns [T, H dv] in u's type."""
     _check(u, "u", (None, None))
     T, ldu = u.shape
     _check(rows, "rows", (T, None), u.dtype)
@@ -1167,7 +1186,7 @@ def delta_rule(u: torch.Tensor, rows: torch.Tensor, cols: Tuple[int, int, int], 
     R = q_start.shape[0]
     for t, nm in ((q_start, "q_start"), (q_len, "q_len"), (slots, "slots")):
         _check(t, nm, (R,), torch.int32)
-    ch, ks, cols = delta_layout(d, dv)
+    ch, ks, cols = delta_layout(d, dv, single_tokens)
     if state_offset + H * dv * ch * ks > state.shape[1]:
         raise KernelError("delta_rule: the state rows are too short")
     out = torch.empty((T, H * dv), dtype=u.dtype, device=u.device)
@@ -1531,13 +1550,17 @@ def wide_launch_shape(n_rows: int, n_heads: int, max_kv: int):
 
 
 def attention_wide(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, row_req: torch.Tensor, positions: torch.Tensor,
-                   block_table: torch.Tensor, window: Optional[int], scale: float, chunk: int, max_splits: int) -> torch.Tensor:
+                   block_table: torch.Tensor, window: Optional[int], scale: float, chunk: int, max_splits: int,
+                   sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal (optionally windowed) attention of q [T, nH, d] over one shared kv head with keys of d and values of dv
     elements (K [pages, 1, page, d], V [pages, 1, dv, page]) on the matrix cores, for widths the other matrix-core kernels
     do not take; returns [T, nH * dv].  Every row's keys are cut into splits of ``chunk`` (``max_splits`` * chunk must
-    reach past the largest position) and merged by a second launch."""
+    reach past the largest position) and merged by a second launch.  ``sinks`` float32 [nH]: a score per head that joins
+    its softmax's denominator."""
     _check(q, "q", (None, None, None), torch.bfloat16)
     T, nH, d = q.shape
+    if sinks is not None:
+        _check(sinks, "sinks", (nH,), torch.float32)
     _check(k_cache, "k_cache", (None, 1, None, d), torch.bfloat16)
     n_pages, _, page_size, _ = k_cache.shape
     _check(v_cache, "v_cache", (n_pages, 1, None, page_size), torch.bfloat16)
@@ -1552,10 +1575,10 @@ def attention_wide(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     part_o = torch.empty((T, nH, max_splits, dv), dtype=torch.float32, device=q.device)
     part_ml = torch.empty((T, nH, max_splits, 2), dtype=torch.float32, device=q.device)
     _call(load_module("attn_wide", (("K_DIM", d), ("V_DIM", dv))), "ifx_attn_wide",
-          (P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, P, P, P),
+          (P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, P, P, P, P),
           q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), 0, row_req.data_ptr(), positions.data_ptr(),
           block_table.data_ptr(), block_table.shape[1], T, nH, d, dv, page_size, int(window or 0), int(chunk), int(max_splits),
-          float(scale), part_o.data_ptr(), part_ml.data_ptr(), _stream())
+          float(scale), part_o.data_ptr(), part_ml.data_ptr(), _ptr(sinks), _stream())
     return out
 
 

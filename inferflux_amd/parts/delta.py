@@ -100,7 +100,7 @@ class GatedDeltaRule(Mixer):
             t.mark("mixer.conv")
         y = ops.delta_rule(u, rows, (C, C + V, C + V + nh), self.A_log, self.dt_bias, self.norm_w, self.norm_eps, nh,
                            self.n_kv_heads, self.head_dim, self.v_head_dim, state, self.conv_floats, ctx.q_start, ctx.q_len,
-                           ctx.state_slots)
+                           ctx.state_slots, single_tokens=ctx.n_tokens == ctx.n_requests)
         if t is not None:
             t.mark("mixer.scan")
         if sink is not None and ops.adds_into_stream(y.shape[0], self.w_o, sink.norm_weight):
