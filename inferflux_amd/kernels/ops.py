@@ -1118,7 +1118,7 @@ def attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 # ----------------------------------------------------------------------------------------
 DELTA_THREAD_CHANNELS = (4, 8, 16, 32, 64)  # key channels of a column of S a thread may hold
 DELTA_MAX_PADDED_DIM, DELTA_MAX_COLS, DELTA_THREADS = 256, 128, 256
-DELTA_DECODE_MAX_CHANNELS = 16              # ... at most this many in steps of single tokens (more would not fit the registers)
+DELTA_DECODE_MAX_CHANNELS = 8               # ... at most this many in steps of single tokens (64 decoded rows at 16 heads of 64 x 128: 62.8 us with 8, 70.2 with 16)
 
 
 def delta_padded_dim(d: int) -> int:
