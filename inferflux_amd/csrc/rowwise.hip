@@ -118,16 +118,19 @@ extern "C" int ifx_sigmoid_gate(const void* x, const void* g, int ld, int g_col,
   IFX_LAUNCH_CHECK();
 }
 
-// One workgroup per row: the row's gate sigmoid(h . w) in float, then out = sum of the base slices + gate * extra.
+// One workgroup per row: the row's gate sigmoid(h . w) in float (1 where w is null), then out = sum of the base slices + gate * extra.
 template <typename T>
 __global__ __launch_bounds__(256) void gated_add_kernel(const void* __restrict__ base, int base_f32, int n_slices, size_t slice_stride,
                                                         const void* __restrict__ extra, int extra_f32, int extra_slices, size_t extra_stride,
                                                         const T* __restrict__ h, const T* __restrict__ w, int K, T* __restrict__ out, int N) {
   __shared__ float red[16];
   const size_t t = blockIdx.x;
-  float z = 0.f;
-  for (int k = threadIdx.x; k < K; k += 256) z = fmaf(to_f(h[t * K + k]), to_f(w[k]), z);
-  const float gate = 1.0f / (1.0f + expf(-block_sum(z, red)));
+  float gate = 1.0f;                 // (without a gate's weight the branch is added as it is)
+  if (w) {
+    float z = 0.f;
+    for (int k = threadIdx.x; k < K; k += 256) z = fmaf(to_f(h[t * K + k]), to_f(w[k]), z);
+    gate = 1.0f / (1.0f + expf(-block_sum(z, red)));
+  }
   for (int c = threadIdx.x; c < N; c += 256) {
     float b;
     if (base_f32) {

@@ -1498,12 +1498,14 @@ def sigmoid_gate(x: torch.Tensor, rows, g_col: int) -> torch.Tensor:
     return out
 
 
-def gated_add(base, extra, h: torch.Tensor, gate_weight: torch.Tensor) -> torch.Tensor:
+def gated_add(base, extra, h: torch.Tensor, gate_weight: Optional[torch.Tensor]) -> torch.Tensor:
     """base + sigmoid(h . gate_weight) * extra row by row: ``base`` and ``extra`` [T, N] (h's type, or ``SliceSums``, which are
-    added in slice order), ``h`` [T, K], ``gate_weight`` [K] (one number per row, formed in float).  Returns [T, N] in h's type."""
+    added in slice order), ``h`` [T, K], ``gate_weight`` [K] (one number per row, formed in float; None: the gate is 1, and
+    ``h`` only says the type and the number of rows).  Returns [T, N] in h's type."""
     _check(h, "h", (None, None))
     T, K = h.shape
-    _check(gate_weight, "gate_weight", (K,), h.dtype)
+    if gate_weight is not None:
+        _check(gate_weight, "gate_weight", (K,), h.dtype)
 
     def operand(v, nm):
         if isinstance(v, SliceSums):
@@ -1518,7 +1520,7 @@ def gated_add(base, extra, h: torch.Tensor, gate_weight: torch.Tensor) -> torch.
         raise KernelError(f"gated_add: base is {N} wide, extra {N2}")
     out = torch.empty((T, N), dtype=h.dtype, device=h.device)
     _call(load_module("rowwise"), "ifx_gated_add", (P, I, I, LL, P, I, I, LL, P, P, I, P, I, I, I, P),
-          bp, bf, bn, bs, ep, ef, en, es, h.data_ptr(), gate_weight.data_ptr(), K, out.data_ptr(), _dt(h), T, N, _stream())
+          bp, bf, bn, bs, ep, ef, en, es, h.data_ptr(), _ptr(gate_weight), K, out.data_ptr(), _dt(h), T, N, _stream())
     return out
 
 

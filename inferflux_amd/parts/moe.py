@@ -126,11 +126,7 @@ class MixtureOfExperts(FeedForward):
         if self.shared is None:
             return out
         extra = self.shared.forward(x, ctx)
-        if self.shared_gate:
-            return ops.gated_add(out, extra, x, self.shared_gate_w)
-        a = out.sum(torch.float32) if isinstance(out, ops.SliceSums) else out.float()
-        b = extra.sum(torch.float32) if isinstance(extra, ops.SliceSums) else extra.float()
-        return (a + b).to(x.dtype)
+        return ops.gated_add(out, extra, x, self.shared_gate_w if self.shared_gate else None)     # (one kernel, also for partial sums)
 
     def forward(self, h, ctx):
         x = h if h.dtype == self.router.dtype else h.to(self.router.dtype)
