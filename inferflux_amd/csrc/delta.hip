@@ -59,14 +59,20 @@ __device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log
 // row of 16 lanes swap through the lanes' own data paths (pairs, quads, mirrored halves of 8, mirrored rows of 16: a few
 // cycles each, where a trip through the LDS crossbar costs a token's whole arithmetic); wider groups go on by shuffles.
 // The order of the additions is fixed by the lane numbers.
-#define DPP_ADD(v, ctrl) (v) += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), (ctrl), 0xF, 0xF, true))
-__device__ __forceinline__ float column_sum(float v, int KS) {
-  if (KS >= 2) DPP_ADD(v, 0xB1);        // quad_perm [1, 0, 3, 2]
-  if (KS >= 4) DPP_ADD(v, 0x4E);        // quad_perm [2, 3, 0, 1]
-  if (KS >= 8) DPP_ADD(v, 0x141);       // row_half_mirror
-  if (KS >= 16) DPP_ADD(v, 0x140);      // row_mirror
-  if (KS >= 32) v += __shfl_xor(v, 16, WAVE);
-  if (KS >= 64) v += __shfl_xor(v, 32, WAVE);
+#define DPP_OF(v, ctrl) __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), (ctrl), 0xF, 0xF, true))
+// f[k] is 1 where the group has more than 2^k lanes and 0 where not: a step the group does not need adds nothing, and the
+// walk has no branches for the steps within a row of 16 lanes.
+struct LaneSteps { float f[4]; int lanes; };
+__device__ __forceinline__ LaneSteps lane_steps(int KS) {
+  return LaneSteps{{KS >= 2 ? 1.f : 0.f, KS >= 4 ? 1.f : 0.f, KS >= 8 ? 1.f : 0.f, KS >= 16 ? 1.f : 0.f}, KS};
+}
+__device__ __forceinline__ float column_sum(float v, const LaneSteps& st) {
+  v = fmaf(st.f[0], DPP_OF(v, 0xB1), v);        // quad_perm [1, 0, 3, 2]
+  v = fmaf(st.f[1], DPP_OF(v, 0x4E), v);        // quad_perm [2, 3, 0, 1]
+  v = fmaf(st.f[2], DPP_OF(v, 0x141), v);       // row_half_mirror
+  v = fmaf(st.f[3], DPP_OF(v, 0x140), v);       // row_mirror
+  if (st.lanes >= 32) v += __shfl_xor(v, 16, WAVE);
+  if (st.lanes >= 64) v += __shfl_xor(v, 32, WAVE);
   return v;
 }
 
@@ -79,7 +85,7 @@ __global__ __launch_bounds__(256) void delta_kernel(DeltaArgs a) {
   // LDS as the head's sizes need it (so that several workgroups share a compute unit): q and k of a stage [STAGE][dpad]
   // each, then its v and o [STAGE][cols] each
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  __shared__ float beta_s[STAGE], g_s[STAGE];
+  __shared__ float beta_s[STAGE + 1], g_s[STAGE + 1];      // (one more: the walk reads a token ahead, also behind the last)
   const int n_cb = (a.dv + a.cols - 1) / a.cols;
   const int h = blockIdx.x / n_cb, j0 = (blockIdx.x % n_cb) * a.cols, r = blockIdx.y;
   const int n = a.q_len[r];
@@ -103,6 +109,7 @@ __global__ __launch_bounds__(256) void delta_kernel(DeltaArgs a) {
   const T* u = (const T*)a.u;
   const T* rows = (const T*)a.rows;
   const float decay_rate = expf(a.A_log[h]), dt_b = a.dt_bias[h], q_mult = 1.0f / sqrtf((float)d);
+  const LaneSteps col_steps = lane_steps(KS);
   const int NL = nthr >= 256 ? 8 : (nthr >= 128 ? 4 : 2);      // lanes to a (token, vector) pair of a stage's 2 STAGE unit norms
   // What a thread fetches of a stage: elements x = tid, tid + nthr, ... of the stage's (token, channel) pairs of q and of k
   // and of its (token, column) pairs of v.  STAGE * dpad and STAGE * cols are at most MAX_PRE * nthr.
@@ -167,13 +174,14 @@ __global__ __launch_bounds__(256) void delta_kernel(DeltaArgs a) {
     if (base + STAGE < n) fetch(base + STAGE);          // the next stage's loads are on their way during the norms and the walk
     // unit norms: NL neighbouring lanes per (token, q or k), all pairs at once; the lanes' squares added by column_sum
     {
+      const LaneSteps norm_steps = lane_steps(NL);
       const int pair = tid / NL, l = tid % NL;
       float* vec = ((pair & 1) ? k_s : q_s) + min(pair >> 1, STAGE - 1) * dpad;
       const bool mine = pair < 2 * cnt;
       float ss = 0.f;
       if (mine)
         for (int c = l; c < d; c += NL) ss = fmaf(vec[c], vec[c], ss);
-      ss = column_sum(ss, NL);
+      ss = column_sum(ss, norm_steps);
       if (mine) {
         const float f = ((pair & 1) ? 1.0f : q_mult) / sqrtf(ss + 1e-6f);
         for (int c = l; c < d; c += NL) vec[c] *= f;
@@ -183,26 +191,31 @@ __global__ __launch_bounds__(256) void delta_kernel(DeltaArgs a) {
     if (owner) {
       // a token's k, q, v, decay and beta are read from LDS while the token before it is worked on; the sums over a
       // thread's channels run in four chains that are added at the end (a fixed order)
-      float kn[CH], qn[CH], vn = v_s[jl], gn = g_s[0], bn = beta_s[0];
+      const float* kp = k_s + s * CH;          // this thread's channels of the stage's first token; a token further: + dpad
+      const float* qp = q_s + s * CH;
+      const float* vp = v_s + jl;
+      float kn[CH], qn[CH], vn = vp[0], gn = g_s[0], bn = beta_s[0];
 #pragma unroll
-      for (int i = 0; i < CH; ++i) { kn[i] = k_s[s * CH + i]; qn[i] = q_s[s * CH + i]; }
+      for (int i = 0; i < CH; ++i) { kn[i] = kp[i]; qn[i] = qp[i]; }
+#pragma unroll 2
       for (int tt = 0; tt < cnt; ++tt) {
         float kk[CH], qq[CH];
         const float gd = gn, bt = bn, vt = vn;
 #pragma unroll
         for (int i = 0; i < CH; ++i) { kk[i] = kn[i]; qq[i] = qn[i]; }
-        if (tt + 1 < cnt) {
-          vn = v_s[(tt + 1) * a.cols + jl]; gn = g_s[tt + 1]; bn = beta_s[tt + 1];
+        // the token after this one, also behind the stage's last, where what is read lies inside the workgroup's LDS all the
+        // same (the row behind q's last is k's first, behind k's last v's first, behind v's last o's first) and is never used
+        kp += dpad; qp += dpad; vp += a.cols;
+        vn = vp[0]; gn = g_s[tt + 1]; bn = beta_s[tt + 1];
 #pragma unroll
-          for (int i = 0; i < CH; ++i) { kn[i] = k_s[(tt + 1) * dpad + s * CH + i]; qn[i] = q_s[(tt + 1) * dpad + s * CH + i]; }
-        }
+        for (int i = 0; i < CH; ++i) { kn[i] = kp[i]; qn[i] = qp[i]; }
         float p4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < CH; ++i) {
           S[i] *= gd;
           p4[i & 3] = fmaf(S[i], kk[i], p4[i & 3]);
         }
-        const float pred = column_sum((p4[0] + p4[1]) + (p4[2] + p4[3]), KS);
+        const float pred = column_sum((p4[0] + p4[1]) + (p4[2] + p4[3]), col_steps);
         const float upd = bt * (vt - pred);
         float o4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -210,7 +223,7 @@ __global__ __launch_bounds__(256) void delta_kernel(DeltaArgs a) {
           S[i] = fmaf(kk[i], upd, S[i]);
           o4[i & 3] = fmaf(S[i], qq[i], o4[i & 3]);
         }
-        const float out = column_sum((o4[0] + o4[1]) + (o4[2] + o4[3]), KS);
+        const float out = column_sum((o4[0] + o4[1]) + (o4[2] + o4[3]), col_steps);
         if (s == 0) o_s[tt * a.cols + jl] = out;
       }
     }
@@ -263,7 +276,7 @@ extern "C" int ifx_delta_rule(const void* u, int ldu, const void* rows, int ldr,
   const int threads = (cols * ks + WAVE - 1) / WAVE * WAVE;
   const dim3 grid(H * ((dv + cols - 1) / cols), R);
   hipStream_t s = (hipStream_t)stream;
-  const size_t lds_bytes = (size_t)2 * STAGE * (ch * ks + cols) * sizeof(float);
+  const size_t lds_bytes = ((size_t)2 * STAGE * (ch * ks + cols) + ch * ks) * sizeof(float);      // (+ a row: the walk reads a token ahead)
 #define LAUNCH(TY, C) hipLaunchKernelGGL((delta_kernel<TY, C>), grid, dim3(threads), lds_bytes, s, a)
 #define BY_CH(TY)                                             \
   do {                                                        \
